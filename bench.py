@@ -1,0 +1,189 @@
+#!/usr/bin/env python3
+"""Benchmark of the paged-decode hot path on one MI355X.
+
+A step is one paged decode attention call (split-K launch + combine launch)
+over one synthetic batch that is already resident in HBM.  The default
+workload is C2 (Qwen3-8B shape: B=64, Hq=32, Hkv=8, D=128, page 256,
+ctx 4096).  One JSON line is printed on stdout.
+
+  value                GB/s = algorithmic bytes per call / mean time per call
+  roofline.achieved    same bytes / mean duration of the split-K kernel alone,
+                       timed with events on the launch stream
+  cpu_baseline         the CPU oracle (a NumPy port of the reference's pure-JAX
+                       paged attention) on a bounded sample of the same batch
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBPS = 8000.0
+
+
+def device_inputs(w, torch, dev):
+    """Seeded N(0,1) bf16 q / K / V drawn on the device, plus the metadata."""
+    g = torch.Generator(device=dev)
+    g.manual_seed(w.seed)
+    shape = (w.num_blocks, w.block_size, w.num_kv_heads, w.head_dim)
+    kc = torch.empty(shape, dtype=torch.bfloat16, device=dev)
+    vc = torch.empty(shape, dtype=torch.bfloat16, device=dev)
+    # page by page keeps the fp32 temporaries small at the multi-GiB configs
+    step = max(1, (1 << 26) // (w.block_size * w.num_kv_heads * w.head_dim))
+    for t in (kc, vc):
+        for p0 in range(0, w.num_blocks, step):
+            n = min(step, w.num_blocks - p0)
+            t[p0:p0 + n] = torch.randn((n,) + shape[1:], generator=g, device=dev,
+                                       dtype=torch.float32).to(torch.bfloat16)
+    q = (torch.randn((w.batch, w.num_heads, w.head_dim), generator=g, device=dev,
+                     dtype=torch.float32) * w.q_gain).to(torch.bfloat16)
+    k_new = torch.randn((w.batch, w.num_kv_heads, w.head_dim), generator=g, device=dev,
+                        dtype=torch.float32)
+    v_new = torch.randn((w.batch, w.num_kv_heads, w.head_dim), generator=g, device=dev,
+                        dtype=torch.float32).to(torch.bfloat16)
+    bt = torch.from_numpy(w.block_tables).to(dev)
+    ctx = torch.from_numpy(w.context_lens).to(dev)
+    slots = torch.from_numpy(w.slot_mapping).to(dev)
+    return q, kc, vc, bt, ctx, slots, k_new, v_new
+
+
+def to_bits(t):
+    import torch
+    return t.detach().cpu().contiguous().view(torch.int16).numpy().view(np.uint16)
+
+
+def timed(fn, steps, torch):
+    """Mean ms per call over `steps` back-to-back calls, from events on the
+    current stream, plus the wall-clock mean."""
+    start = torch.cuda.Event(enable_timing=True)
+    end = torch.cuda.Event(enable_timing=True)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    start.record()
+    for _ in range(steps):
+        fn()
+    end.record()
+    torch.cuda.synchronize()
+    t1 = time.perf_counter()
+    return start.elapsed_time(end) / steps, (t1 - t0) * 1e3 / steps
+
+
+def cpu_baseline(w, q, kc, vc, budget_s=20.0):
+    """Oracle on the host cores over the first sequences of the batch until
+    the time budget is used; extrapolated linearly in live positions."""
+    from oracle.paged_attention_oracle import paged_decode_attention_per_seq_ref
+    from nanovllm_jax_amd.workloads import algorithmic_bytes
+    qb, kb, vb = to_bits(q), to_bits(kc), to_bits(vc)
+    done_pos, done_seq, t_used = 0, 0, 0.0
+    b = 0
+    while b < w.batch and t_used < budget_s:
+        n = min(4, w.batch - b)
+        t0 = time.perf_counter()
+        paged_decode_attention_per_seq_ref(qb[b:b + n], kb, vb, w.block_tables[b:b + n],
+                                           w.context_lens[b:b + n], w.scale, w.block_size)
+        t_used += time.perf_counter() - t0
+        done_pos += int(w.context_lens[b:b + n].sum())
+        done_seq += n
+        b += n
+    byts = algorithmic_bytes(w.context_lens[:done_seq], done_seq, w.num_heads, w.num_kv_heads,
+                             w.head_dim, w.max_blocks)
+    return {"value": round(byts / t_used / 1e9, 4), "unit": "GB/s", "cores": 1, "kind": "port",
+            "us_per_call_extrapolated": round(
+                t_used / max(done_pos, 1) * int(w.context_lens.sum()) * 1e6, 1),
+            "sample": f"NumPy oracle (single thread) on the first {done_seq} of {w.batch} "
+                      f"sequences of {w.name} ({done_pos} positions, {t_used:.1f} s)"}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--workload", default="C2", choices=["C1", "C2", "C3", "C4", "C5"])
+    ap.add_argument("--chunk", type=int, default=0, help="positions per workgroup (0 = default)")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--cpu-budget", type=float, default=20.0)
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build runs on ONE GPU only (the path shards with no exchange "
+              "step; see DESIGN.md); --gpus must be 1", file=sys.stderr)
+        return 2
+
+    import torch
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible; the paged-decode path has no CPU implementation",
+              file=sys.stderr)
+        return 1
+    from nanovllm_jax_amd import _lib, paged_attention, store_kv_to_cache
+    from nanovllm_jax_amd.layers.paged_attention import (default_chunk,
+                                                         paged_decode_workspace_bytes)
+    from nanovllm_jax_amd.workloads import algorithmic_bytes, make_workload
+
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    w = make_workload(args.workload)
+    q, kc, vc, bt, ctx, slots, k_new, v_new = device_inputs(w, torch, dev)
+    chunk = args.chunk or default_chunk(w.batch, w.num_kv_heads, w.max_blocks, w.block_size)
+    ws = torch.empty(paged_decode_workspace_bytes(w.batch, w.num_heads, w.head_dim, w.max_blocks,
+                                                  w.block_size, w.num_kv_heads, chunk),
+                     dtype=torch.uint8, device=dev)
+    out = torch.empty_like(q)
+    kflat = kc.view(-1, w.num_kv_heads, w.head_dim)
+    vflat = vc.view(-1, w.num_kv_heads, w.head_dim)
+
+    def decode(phases=3):
+        paged_attention(q, kc, vc, bt, ctx, w.scale, w.block_size, chunk=chunk, out=out,
+                        workspace=ws, phases=phases)
+
+    def store():
+        store_kv_to_cache(k_new, v_new, kflat, vflat, slots)
+
+    store()
+    for _ in range(args.warmup):
+        decode()
+    ms_call, ms_wall = timed(decode, args.steps, torch)
+    ms_splitk, _ = timed(lambda: decode(_lib.NVJ_PHASE_SPLITK), args.steps, torch)
+    ms_combine, _ = timed(lambda: decode(_lib.NVJ_PHASE_COMBINE), args.steps, torch)
+    ms_store, _ = timed(store, args.steps, torch)
+
+    byts = algorithmic_bytes(w.context_lens, w.batch, w.num_heads, w.num_kv_heads, w.head_dim,
+                             w.max_blocks)
+    gbps = byts / (ms_call * 1e-3) / 1e9
+    gbps_kernel = byts / (ms_splitk * 1e-3) / 1e9
+    rec = {
+        "metric": "paged decode attn HBM GB/s (us/call alongside), Qwen3-8B shape B=64 ctx4k"
+                  if w.name == "C2" else f"paged decode attn HBM GB/s, workload {w.name}",
+        "value": round(gbps, 1), "unit": "GB/s", "n_gpus": 1, "steps": args.steps,
+        "warmup": args.warmup, "ms_per_step": round(ms_wall, 5), "higher_is_better": True,
+        "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
+        "us_per_call": round(ms_call * 1e3, 2),
+        "pct_of_hbm_peak": round(100.0 * gbps / HBM_PEAK_GBPS, 2),
+        "config": {"workload": f"{w.name}: B={w.batch} Hq={w.num_heads} Hkv={w.num_kv_heads} "
+                               f"D={w.head_dim} page={w.block_size} "
+                               f"ctx={int(w.context_lens.min())}..{int(w.context_lens.max())} "
+                               f"pool={w.num_blocks} pages",
+                   "chunk": chunk, "algorithmic_bytes_per_call": byts,
+                   "step": "split-K launch + combine launch"},
+        "roofline": {"bound": "hbm", "achieved": round(gbps_kernel, 1), "peak": HBM_PEAK_GBPS,
+                     "unit": "GB/s", "frac": round(gbps_kernel / HBM_PEAK_GBPS, 4),
+                     "traffic": None, "kernel": "paged_decode_splitk_kernel",
+                     "kernel_us": round(ms_splitk * 1e3, 2)},
+        "other_kernels_us": {"paged_decode_combine_kernel": round(ms_combine * 1e3, 2),
+                             "store_kvcache_kernel": round(ms_store * 1e3, 2)},
+    }
+    if not args.no_cpu_baseline:
+        rec["cpu_baseline"] = cpu_baseline(w, q, kc, vc, args.cpu_budget)
+    print(json.dumps(rec), flush=True)
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

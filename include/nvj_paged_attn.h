@@ -1,0 +1,152 @@
+/*
+ * C ABI of the MI355X (gfx950) paged-decode path: KV-cache store and split-K
+ * paged decode attention.
+ *
+ * Every entry point takes plain device pointers, sizes and a HIP stream
+ * (passed as void* so the header needs no HIP include), only ENQUEUES work on
+ * that stream, never synchronises, never allocates, keeps no global mutable
+ * state and is re-entrant.  Return value: 0 on success, a negative NVJ_ERR_*
+ * code otherwise (never throws, never exits).  Citations name the reference
+ * interface each entry point stands in for (paths relative to the reference
+ * checkout).
+ */
+#ifndef NVJ_PAGED_ATTN_H_
+#define NVJ_PAGED_ATTN_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define NVJ_ABI_VERSION 1
+
+/* exported from the shared library (which is built with hidden visibility) */
+#define NVJ_API __attribute__((visibility("default")))
+
+/* error codes */
+#define NVJ_OK                 0
+#define NVJ_ERR_NULL_POINTER  -1   /* a required pointer is NULL                    */
+#define NVJ_ERR_BAD_SHAPE     -2   /* negative size, Hq % Hkv != 0, ...             */
+#define NVJ_ERR_UNSUPPORTED   -3   /* head_dim / group size / block size not built  */
+#define NVJ_ERR_WORKSPACE     -4   /* workspace too small or misaligned             */
+#define NVJ_ERR_LAUNCH        -5   /* hipGetLastError() != hipSuccess after launch  */
+#define NVJ_ERR_BAD_DTYPE     -6   /* unknown element type code                     */
+
+/* element type codes for the new K/V rows handed to the store */
+#define NVJ_DTYPE_BF16 0
+#define NVJ_DTYPE_F32  1
+
+/* Human-readable text for an NVJ_ERR_* code (static storage). */
+NVJ_API const char* nvj_error_string(int code);
+
+/* NVJ_ABI_VERSION the library was built with. */
+NVJ_API int nvj_abi_version(void);
+
+/*
+ * KV-cache store.  Replaces store_kv_to_cache (layers/attention.py:42-77) as
+ * called from Attention.__call__ on the flattened cache
+ * (layers/attention.py:457-475).
+ *
+ *   key   [num_tokens, num_kv_heads, head_dim]  k_dtype (bf16 or f32; the
+ *         reference hands over f32 keys after RoPE and casts, :70)
+ *   value [num_tokens, num_kv_heads, head_dim]  v_dtype
+ *   k_cache, v_cache [num_slots, num_kv_heads, head_dim] bf16, updated IN PLACE
+ *         (num_slots = num_blocks * block_size)
+ *   slot_mapping [num_tokens] int32
+ *
+ * cache[slot[i]] = bf16_round_nearest_even(x[i]) for 0 <= slot[i] < num_slots;
+ * slot[i] >= num_slots is dropped (mode='drop', :74); slot[i] < 0 is SKIPPED
+ * (the documented meaning of -1, :57-58 -- the reference's code would write
+ * row 0 instead).  Rows not named by slot_mapping are not touched.  Duplicate
+ * slots: one of the writers wins, unspecified which (as in the reference).
+ * num_tokens == 0 is a no-op.  head_dim * num_kv_heads must be a multiple of 8.
+ */
+NVJ_API int nvj_store_kvcache_launch(void* stream,
+                             const void* key, const void* value,
+                             void* k_cache, void* v_cache,
+                             const int32_t* slot_mapping,
+                             int32_t num_tokens, int32_t num_kv_heads,
+                             int32_t head_dim, int64_t num_slots,
+                             int32_t k_dtype, int32_t v_dtype);
+
+/*
+ * Split size (positions of one sequence handled by one workgroup) the library
+ * would pick for this problem when the caller passes chunk == 0.  Always a
+ * multiple of 32.
+ */
+NVJ_API int32_t nvj_paged_decode_default_chunk(int32_t batch, int32_t num_kv_heads,
+                                       int32_t max_blocks, int32_t block_size);
+
+/*
+ * Bytes of device workspace nvj_paged_decode_launch needs for the split-K
+ * partials (fp32 accumulators plus running max and sum per split).  chunk == 0
+ * means the default chunk.  Returns 0 on invalid arguments.
+ */
+NVJ_API size_t nvj_paged_decode_workspace_bytes(int32_t batch, int32_t num_heads,
+                                        int32_t head_dim, int32_t max_blocks,
+                                        int32_t block_size, int32_t num_kv_heads,
+                                        int32_t chunk);
+
+/*
+ * Paged decode attention, one query position per sequence.  Replaces
+ * paged_attention (layers/pallas_attention.py:465-507) ->
+ * paged_decode_attention_vectorized (:146-238) as dispatched from
+ * Attention._decode_attention (layers/attention.py:389-397), and equally the
+ * gather + dot_product_attention fallback (layers/attention.py:399-434).
+ *
+ *   q            [batch, num_heads, head_dim]                         bf16
+ *   k_cache, v_cache [num_blocks, block_size, num_kv_heads, head_dim] bf16
+ *   block_tables [batch, max_blocks] int32; entries at or beyond
+ *                ceil(context_lens[b] / block_size) are never read (the
+ *                reference pads them with -1, engine/model_runner.py:240)
+ *   context_lens [batch] int32 (counts the position being decoded,
+ *                engine/model_runner.py:360)
+ *   out          [batch, num_heads, head_dim]                         bf16
+ *   workspace    >= nvj_paged_decode_workspace_bytes(...) bytes, 16-byte aligned,
+ *                contents need not be initialised
+ *
+ * out[b,h,:] = softmax_{s < ctx[b]}(scale * q[b,h,:] . K[b,s,h/G,:]) V[b,s,h/G,:]
+ * with G = num_heads / num_kv_heads, fp32 accumulation, bf16 result.
+ * context_lens[b] <= 0 gives a row of zeros (0 / (0 + 1e-9), :227).  Positions
+ * >= context_lens[b] are never read.  Table entries of live pages must lie in
+ * [0, num_blocks); the kernel clamps them into range like the reference (:185)
+ * rather than faulting.
+ *
+ * Two launches on `stream`: the split-K kernel (one workgroup per
+ * (sequence, chunk of positions), all KV heads) and the combine pass.
+ * Supported: head_dim 128, num_heads / num_kv_heads <= 16, block_size a
+ * multiple of 32, chunk a multiple of 32 (0 = default).
+ */
+NVJ_API int nvj_paged_decode_launch(void* stream,
+                            const void* q, const void* k_cache, const void* v_cache,
+                            const int32_t* block_tables, const int32_t* context_lens,
+                            void* out, void* workspace, size_t workspace_bytes,
+                            int32_t batch, int32_t num_heads, int32_t num_kv_heads,
+                            int32_t head_dim, int32_t block_size, int32_t max_blocks,
+                            int32_t num_blocks, float scale, int32_t chunk);
+
+/*
+ * The same call with its two launches selectable: NVJ_PHASE_SPLITK runs the
+ * split-K kernel only (partials stay in `workspace`), NVJ_PHASE_COMBINE the
+ * combine pass only (reads the partials an earlier split-K launch with the
+ * same arguments left in `workspace`).  Both bits = nvj_paged_decode_launch.
+ * For timing one launch in isolation and for callers that want other work
+ * between the two; same reference counterpart as nvj_paged_decode_launch.
+ */
+#define NVJ_PHASE_SPLITK  1u
+#define NVJ_PHASE_COMBINE 2u
+NVJ_API int nvj_paged_decode_launch_phases(void* stream,
+                            const void* q, const void* k_cache, const void* v_cache,
+                            const int32_t* block_tables, const int32_t* context_lens,
+                            void* out, void* workspace, size_t workspace_bytes,
+                            int32_t batch, int32_t num_heads, int32_t num_kv_heads,
+                            int32_t head_dim, int32_t block_size, int32_t max_blocks,
+                            int32_t num_blocks, float scale, int32_t chunk,
+                            uint32_t phases);
+
+#ifdef __cplusplus
+}  /* extern "C" */
+#endif
+#endif  /* NVJ_PAGED_ATTN_H_ */

@@ -1,0 +1,11 @@
+"""MI355X-native paged-decode path: KV-cache store + split-K paged decode attention.
+
+Importing the package does not load the HIP library; the first call does, and
+fails loudly if it has not been built.
+"""
+from .layers.attention import Attention, store_kv_to_cache
+from .layers.paged_attention import paged_attention
+from .utils.context import AttentionContext, create_decode_context
+
+__all__ = ["Attention", "store_kv_to_cache", "paged_attention", "AttentionContext",
+           "create_decode_context"]

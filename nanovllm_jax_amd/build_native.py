@@ -1,0 +1,59 @@
+"""Compile the HIP kernels and their C ABI into one shared library for gfx950.
+
+``hipcc`` cross-compiles without a GPU.  The library is built in-tree
+(``nanovllm_jax_amd/_native/libnvj_paged_attn.so``) so that it travels with the
+source tree; nothing here runs at import time of the package.
+"""
+from __future__ import annotations
+
+import os
+import shutil
+import subprocess
+import sys
+
+PKG_DIR = os.path.dirname(os.path.abspath(__file__))
+REPO_DIR = os.path.dirname(PKG_DIR)
+CSRC_DIR = os.path.join(PKG_DIR, "csrc")
+NATIVE_DIR = os.path.join(PKG_DIR, "_native")
+LIB_NAME = "libnvj_paged_attn.so"
+LIB_PATH = os.path.join(NATIVE_DIR, LIB_NAME)
+
+SOURCES = ("store_kvcache.hip", "paged_decode.hip")
+
+HIPCC_FLAGS = (
+    "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-shared",
+    "-fvisibility=hidden", "-Wall", "-Wno-unused-function",
+    # packed fp32 VALU forms are kept out of the generated code
+    "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+)
+
+
+def hipcc_path() -> str:
+    for cand in (os.environ.get("HIPCC"), shutil.which("hipcc"), "/opt/rocm/bin/hipcc"):
+        if cand and os.path.exists(cand):
+            return cand
+    raise RuntimeError("hipcc not found (set HIPCC or put /opt/rocm/bin on PATH)")
+
+
+def build(verbose: bool = True, extra_flags: tuple[str, ...] = ()) -> str:
+    """Compile every HIP source into ``LIB_PATH`` (always recompiles)."""
+    os.makedirs(NATIVE_DIR, exist_ok=True)
+    tmp = LIB_PATH + ".tmp"
+    cmd = [hipcc_path(), *HIPCC_FLAGS, *extra_flags,
+           "-I", os.path.join(REPO_DIR, "include"),
+           *[os.path.join(CSRC_DIR, s) for s in SOURCES], "-o", tmp]
+    if verbose:
+        print("[build]", " ".join(cmd), flush=True)
+    proc = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    out = "\n".join(l for l in proc.stdout.splitlines()
+                    if "packed-fp32-ops' is not a recognized feature" not in l)
+    if proc.returncode != 0:
+        raise RuntimeError(f"hipcc failed ({proc.returncode}):\n{out}")
+    if verbose and out.strip():
+        print(out, flush=True)
+    os.replace(tmp, LIB_PATH)
+    return LIB_PATH
+
+
+if __name__ == "__main__":
+    print(build(extra_flags=tuple(sys.argv[1:])))

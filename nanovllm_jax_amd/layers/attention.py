@@ -1,0 +1,114 @@
+"""Attention layer over a block-paged KV cache: store, then decode.
+
+Host-side mirror of ``layers/attention.py`` of the reference for the decode
+phase: ``store_kv_to_cache`` (:42-77) and ``Attention`` (:282-480) keep their
+names, argument order and return shapes.  Both run on the HIP library only;
+there is no prefill here (``context.is_prefill=True`` raises) and no alternate
+dispatch.
+
+Differences a caller can observe, both deliberate:
+* the cache is updated in place and the very same tensors are returned (the
+  reference returns new arrays that alias the donated inputs);
+* a negative slot stores nothing (the reference's docstring, :57-58; its code
+  writes row 0 instead).
+"""
+from __future__ import annotations
+
+import torch
+
+from .. import _lib
+from ..utils.context import AttentionContext
+from .paged_attention import paged_attention
+
+__all__ = ["store_kv_to_cache", "Attention"]
+
+_DTYPE_CODE = {torch.bfloat16: _lib.NVJ_DTYPE_BF16, torch.float32: _lib.NVJ_DTYPE_F32}
+
+
+def _require(cond: bool, msg: str) -> None:
+    if not cond:
+        raise ValueError(msg)
+
+
+def store_kv_to_cache(key, value, k_cache, v_cache, slot_mapping):
+    """Scatter new K/V rows into the paged cache through ``slot_mapping``.
+
+    key, value   [num_tokens, num_kv_heads, head_dim], bf16 or float32 (float32
+                 rows are rounded to nearest-even bf16, as ``astype`` does)
+    k_cache, v_cache
+                 [num_slots, num_kv_heads, head_dim] bf16, or the 4-D
+                 [num_blocks, block_size, num_kv_heads, head_dim] view of the
+                 same memory
+    slot_mapping [num_tokens] int32; ``slot < 0`` skips the token, ``slot >=
+                 num_slots`` drops it
+
+    Returns ``(k_cache, v_cache)``: the tensors passed in, updated in place.
+    """
+    lib = _lib.load()
+    for name, t in (("key", key), ("value", value), ("k_cache", k_cache),
+                    ("v_cache", v_cache), ("slot_mapping", slot_mapping)):
+        _require(isinstance(t, torch.Tensor), f"{name} must be a torch.Tensor")
+        _require(t.is_cuda, f"{name} must live on the GPU (got {t.device}); "
+                            "the KV-cache store has no CPU implementation")
+        _require(t.is_contiguous(), f"{name} must be contiguous")
+        _require(t.device == key.device, f"{name} is on {t.device}, key on {key.device}")
+    _require(key.dim() == 3 and value.shape == key.shape,
+             "key and value must both be [num_tokens, num_kv_heads, head_dim]")
+    _require(key.dtype in _DTYPE_CODE, f"key dtype {key.dtype} not supported")
+    _require(value.dtype in _DTYPE_CODE, f"value dtype {value.dtype} not supported")
+    _require(k_cache.dtype == torch.bfloat16 and v_cache.dtype == torch.bfloat16,
+             "caches must be bf16")
+    _require(k_cache.shape == v_cache.shape and k_cache.dim() in (3, 4),
+             "caches must have equal 3-D or 4-D shapes")
+    num_tokens, num_kv_heads, head_dim = key.shape
+    _require(tuple(k_cache.shape[-2:]) == (num_kv_heads, head_dim),
+             f"cache rows {tuple(k_cache.shape[-2:])} != key rows {(num_kv_heads, head_dim)}")
+    _require(slot_mapping.dtype == torch.int32 and slot_mapping.shape == (num_tokens,),
+             "slot_mapping must be int32 [num_tokens]")
+    num_slots = k_cache.numel() // (num_kv_heads * head_dim)
+    with torch.cuda.device(key.device):
+        stream = torch.cuda.current_stream(key.device).cuda_stream
+        code = lib.nvj_store_kvcache_launch(
+            stream, key.data_ptr(), value.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(),
+            slot_mapping.data_ptr(), num_tokens, num_kv_heads, head_dim, num_slots,
+            _DTYPE_CODE[key.dtype], _DTYPE_CODE[value.dtype])
+    _lib.check(code, "nvj_store_kvcache_launch")
+    return k_cache, v_cache
+
+
+class Attention:
+    """Multi-head attention with a paged KV cache, decode phase.
+
+    Same constructor and call contract as the reference's ``Attention``
+    (``layers/attention.py:307-329, 436-480``): ``set_kv_cache`` hands over the
+    per-layer ``[num_blocks, block_size, num_kv_heads, head_dim]`` bf16 caches;
+    ``__call__(q, k, v, context)`` first stores the new K/V rows, then attends
+    over the cache (the new row included: ``context_lens`` already counts it).
+    """
+
+    def __init__(self, num_heads: int, head_dim: int, scale: float, num_kv_heads: int,
+                 block_size: int = 256):
+        self.num_heads = num_heads
+        self.head_dim = head_dim
+        self.scale = scale
+        self.num_kv_heads = num_kv_heads
+        self.block_size = block_size
+        self.k_cache = None
+        self.v_cache = None
+
+    def set_kv_cache(self, k_cache, v_cache):
+        self.k_cache = k_cache
+        self.v_cache = v_cache
+
+    def _decode_attention(self, q, context: AttentionContext):
+        q = q.to(self.k_cache.dtype)      # layers/attention.py:386-387
+        return paged_attention(q, self.k_cache, self.v_cache, context.block_tables,
+                               context.context_lens, self.scale, self.block_size)
+
+    def __call__(self, q, k, v, context: AttentionContext):
+        if self.k_cache is None or self.v_cache is None:
+            raise RuntimeError("set_kv_cache() must be called before the first decode step")
+        if context.is_prefill:
+            raise NotImplementedError("this package implements the decode phase only")
+        store_kv_to_cache(k, v, self.k_cache, self.v_cache, context.slot_mapping)
+        return self._decode_attention(q, context)

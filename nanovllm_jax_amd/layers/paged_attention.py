@@ -1,0 +1,111 @@
+"""Paged decode attention entry point.
+
+Host-side mirror of ``paged_attention`` (``layers/pallas_attention.py:465-507``
+of the reference): same positional contract
+``(q, k_cache, v_cache, block_tables, context_lens, scale, block_size)`` and the
+same result shape/dtype, with one dispatch target only: the HIP split-K kernel
+behind ``nvj_paged_decode_launch``.  Tensors are device memory handles
+(``torch`` on ROCm); all arithmetic happens in the HIP library.
+"""
+from __future__ import annotations
+
+import torch
+
+from .. import _lib
+
+__all__ = ["paged_attention", "paged_decode_workspace_bytes", "default_chunk"]
+
+
+def _require(cond: bool, msg: str) -> None:
+    if not cond:
+        raise ValueError(msg)
+
+
+def _check_device_tensor(t: torch.Tensor, name: str, dtype: torch.dtype, ndim: int) -> None:
+    _require(isinstance(t, torch.Tensor), f"{name} must be a torch.Tensor")
+    _require(t.is_cuda, f"{name} must live on the GPU (got {t.device}); "
+                        "the paged-decode path has no CPU implementation")
+    _require(t.dtype == dtype, f"{name} must be {dtype}, got {t.dtype}")
+    _require(t.dim() == ndim, f"{name} must have {ndim} dims, got shape {tuple(t.shape)}")
+    _require(t.is_contiguous(), f"{name} must be contiguous")
+
+
+def default_chunk(batch: int, num_kv_heads: int, max_blocks: int, block_size: int) -> int:
+    """Positions per workgroup the library picks when ``chunk=0``."""
+    return int(_lib.load().nvj_paged_decode_default_chunk(batch, num_kv_heads,
+                                                          max_blocks, block_size))
+
+
+def paged_decode_workspace_bytes(batch: int, num_heads: int, head_dim: int,
+                                 max_blocks: int, block_size: int, num_kv_heads: int,
+                                 chunk: int = 0) -> int:
+    """Bytes of split-K workspace one call needs."""
+    return int(_lib.load().nvj_paged_decode_workspace_bytes(
+        batch, num_heads, head_dim, max_blocks, block_size, num_kv_heads, chunk))
+
+
+def paged_attention(q, k_cache, v_cache, block_tables, context_lens, scale, block_size,
+                    *, chunk: int = 0, out: torch.Tensor | None = None,
+                    workspace: torch.Tensor | None = None,
+                    phases: int = _lib.NVJ_PHASE_SPLITK | _lib.NVJ_PHASE_COMBINE) -> torch.Tensor:
+    """Decode attention over a block-paged KV cache.
+
+    q            [batch, num_heads, head_dim]                          bf16
+    k_cache      [num_blocks, block_size, num_kv_heads, head_dim]      bf16
+    v_cache      same shape
+    block_tables [batch, max_blocks] int32 (padding entries are never read)
+    context_lens [batch] int32
+    scale        softmax scale (Python float)
+    block_size   positions per page; must equal ``k_cache.shape[1]``
+
+    Returns [batch, num_heads, head_dim] bf16.  ``chunk`` (positions per
+    workgroup, multiple of 32, 0 = library default), ``out`` and ``workspace``
+    (uint8 tensor of at least ``paged_decode_workspace_bytes`` bytes) are
+    optional tuning/reuse knobs the reference does not have; ``phases`` selects
+    the split-K launch, the combine launch or both (timing aid).
+    """
+    lib = _lib.load()
+    _check_device_tensor(q, "q", torch.bfloat16, 3)
+    _check_device_tensor(k_cache, "k_cache", torch.bfloat16, 4)
+    _check_device_tensor(v_cache, "v_cache", torch.bfloat16, 4)
+    _check_device_tensor(block_tables, "block_tables", torch.int32, 2)
+    _check_device_tensor(context_lens, "context_lens", torch.int32, 1)
+    batch, num_heads, head_dim = q.shape
+    num_blocks, bs, num_kv_heads, d2 = k_cache.shape
+    _require(v_cache.shape == k_cache.shape, "k_cache and v_cache shapes differ")
+    _require(d2 == head_dim, f"head_dim mismatch: q {head_dim}, cache {d2}")
+    _require(int(block_size) == bs, f"block_size {block_size} != k_cache.shape[1] {bs}")
+    _require(block_tables.shape[0] == batch, "block_tables batch mismatch")
+    _require(context_lens.shape[0] == batch, "context_lens batch mismatch")
+    _require(num_heads % num_kv_heads == 0, "num_heads must be a multiple of num_kv_heads")
+    max_blocks = block_tables.shape[1]
+    dev = q.device
+    for name, t in (("k_cache", k_cache), ("v_cache", v_cache),
+                    ("block_tables", block_tables), ("context_lens", context_lens)):
+        _require(t.device == dev, f"{name} is on {t.device}, q on {dev}")
+
+    if out is None:
+        out = torch.empty_like(q)
+    else:
+        _check_device_tensor(out, "out", torch.bfloat16, 3)
+        _require(out.shape == q.shape and out.device == dev, "out must match q")
+    need = int(lib.nvj_paged_decode_workspace_bytes(batch, num_heads, head_dim, max_blocks,
+                                                    bs, num_kv_heads, chunk)) if batch and max_blocks else 0
+    if workspace is None:
+        workspace = torch.empty(max(need, 16), dtype=torch.uint8, device=dev)
+    else:
+        _require(workspace.is_cuda and workspace.device == dev and workspace.is_contiguous(),
+                 "workspace must be a contiguous tensor on q's device")
+        _require(workspace.numel() * workspace.element_size() >= need,
+                 f"workspace too small: need {need} bytes")
+    ws_bytes = workspace.numel() * workspace.element_size()
+
+    with torch.cuda.device(dev):
+        stream = torch.cuda.current_stream(dev).cuda_stream
+        code = lib.nvj_paged_decode_launch_phases(
+            stream, q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(),
+            block_tables.data_ptr(), context_lens.data_ptr(), out.data_ptr(),
+            workspace.data_ptr(), ws_bytes, batch, num_heads, num_kv_heads, head_dim, bs,
+            max_blocks, num_blocks, float(scale), int(chunk), int(phases))
+    _lib.check(code, "nvj_paged_decode_launch_phases")
+    return out

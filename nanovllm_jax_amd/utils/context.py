@@ -1,0 +1,45 @@
+"""Attention metadata carrier for the decode path.
+
+Host-side mirror of ``utils/context.py`` of the reference (``AttentionContext``
+:35-81, ``create_decode_context`` :169-190): same field names and meaning, with
+device tensors in place of JAX arrays.  Only the decode fields are populated by
+this package; the prefill fields exist so that code written against the
+reference's dataclass keeps working.
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass
+from typing import Any
+
+__all__ = ["AttentionContext", "create_decode_context"]
+
+
+@dataclass
+class AttentionContext:
+    """Metadata one attention call needs.
+
+    is_prefill          False for decode (the only phase this package runs).
+    context_lens        [batch] int32, length of every sequence including the
+                        position being decoded.
+    slot_mapping        [num_tokens] int32, cache slot of every new K/V row;
+                        -1 means "do not store".
+    block_tables        [batch, max_blocks] int32, logical -> physical page,
+                        padded with -1.
+    """
+    is_prefill: bool = False
+    cu_seqlens_q: Any = None
+    cu_seqlens_k: Any = None
+    max_seqlen_q: int = 0
+    max_seqlen_k: int = 0
+    context_lens: Any = None
+    slot_mapping: Any = None
+    block_tables: Any = None
+    last_token_indices: Any = None
+
+
+def create_decode_context(context_lens, slot_mapping, block_tables) -> AttentionContext:
+    """Context for one decode step (every token is a sequence's last token, so
+    ``last_token_indices`` stays None)."""
+    return AttentionContext(is_prefill=False, context_lens=context_lens,
+                            slot_mapping=slot_mapping, block_tables=block_tables,
+                            last_token_indices=None)

@@ -1,0 +1,296 @@
+"""NumPy restatement of the reference's KV-cache store and paged decode attention.
+
+TEST INFRASTRUCTURE ONLY: imported by ``tests/``, ``__graft_entry__.smoke()``
+and ``bench.py``'s ``cpu_baseline`` leg as the checker; never by the product
+package, which has no CPU path.
+
+bf16 tensors are carried as ``uint16`` bit patterns (NumPy has no bf16), fp32
+tensors as ``float32``.  Every function names the reference lines it follows
+(paths relative to the reference checkout).
+
+What pins each function (see tests/test_oracle_pinning.py):
+
+* ``f32_to_bf16_bits``          - IEEE round-to-nearest-even; cross-checked
+                                  against ``torch.Tensor.to(torch.bfloat16)``.
+* ``store_kv_to_cache_ref``     - brute-force per-token Python loop; untouched
+                                  rows unchanged; idempotence; K/V independence.
+* ``paged_decode_attention_vectorized_ref`` and ``..._per_seq``
+                                - fp64 textbook softmax(qK^T)V on small shapes,
+                                  ``torch.nn.functional.scaled_dot_product_attention``
+                                  with ``enable_gqa`` on gathered pages,
+                                  closed forms (ctx=1 -> V row, equal keys ->
+                                  mean of V, ctx=0 -> zeros), permutation and
+                                  padding invariance.
+* ``paged_attention_fallback_ref``
+                                - same checks; the bf16 rounding of the
+                                  probabilities inside ``jax.nn.dot_product_attention``
+                                  (third-party jax, not under the reference
+                                  tree, ``requirements.txt`` pins ``jax>=0.4.20``)
+                                  is restated from its published XLA
+                                  implementation: PARITY UNPINNED at bit level
+                                  for that one rounding step; it is covered by
+                                  the 1e-2 tolerance, not by a vector.
+"""
+from __future__ import annotations
+
+import numpy as np
+
+__all__ = [
+    "f32_to_bf16_bits",
+    "bf16_bits_to_f32",
+    "store_kv_to_cache_ref",
+    "gather_kv_from_cache_ref",
+    "paged_decode_attention_vectorized_ref",
+    "paged_decode_attention_per_seq_ref",
+    "paged_attention_fallback_ref",
+    "textbook_attention_f64",
+]
+
+
+# ---------------------------------------------------------------------------
+# bf16 <-> fp32 on bit patterns
+# ---------------------------------------------------------------------------
+
+def f32_to_bf16_bits(x: np.ndarray) -> np.ndarray:
+    """fp32 -> bf16 bit pattern, round-to-nearest-even (what ``astype(bfloat16)``
+    does in ``layers/attention.py:70-71`` and ``pallas_attention.py:238``).
+    NaN stays a quiet NaN."""
+    x = np.ascontiguousarray(x, dtype=np.float32)
+    u = x.view(np.uint32)
+    rounding_bias = ((u >> np.uint32(16)) & np.uint32(1)) + np.uint32(0x7FFF)
+    r = ((u + rounding_bias) >> np.uint32(16)).astype(np.uint16)
+    nan = np.isnan(x)
+    if nan.any():
+        r = np.where(nan, ((u >> np.uint32(16)) | np.uint32(0x0040)).astype(np.uint16), r)
+    return r
+
+
+def bf16_bits_to_f32(b: np.ndarray) -> np.ndarray:
+    """bf16 bit pattern -> fp32 (exact)."""
+    b = np.ascontiguousarray(b, dtype=np.uint16)
+    return (b.astype(np.uint32) << np.uint32(16)).view(np.float32)
+
+
+def _as_bf16_bits(x: np.ndarray) -> np.ndarray:
+    """Accept fp32 values or uint16 bf16 bits; return bf16 bits."""
+    if x.dtype == np.uint16:
+        return x
+    if x.dtype == np.float32:
+        return f32_to_bf16_bits(x)
+    raise TypeError(f"expected float32 values or uint16 bf16 bits, got {x.dtype}")
+
+
+# ---------------------------------------------------------------------------
+# KV-cache store
+# ---------------------------------------------------------------------------
+
+def store_kv_to_cache_ref(key, value, k_cache, v_cache, slot_mapping,
+                          negative_slots: str = "reference"):
+    """Restates ``store_kv_to_cache`` (``layers/attention.py:42-77``).
+
+    key, value : [T, Hkv, D] float32 values or uint16 bf16 bits
+    k_cache, v_cache : [num_slots, Hkv, D] uint16 bf16 bits (flattened cache,
+                 ``layers/attention.py:458-463``)
+    slot_mapping : [T] int32
+
+    Returns new ``(k_cache, v_cache)``; inputs are not modified (the reference
+    is functional).
+
+    ``negative_slots``:
+      "reference" - what the code does: ``safe = where(slot >= 0, slot, 0)``
+                    (:64-67) then ``.at[safe].set(x, mode='drop')`` (:74-75),
+                    i.e. a negative slot WRITES ROW 0; slots >= num_slots are
+                    dropped.  Duplicate targets have no defined winner in XLA;
+                    here the last writer wins.
+      "skip"      - what the docstring (:57-58) and ``utils/context.py:57-58``
+                    promise ("-1 indicates skip"): negative slots write nothing.
+                    This is the contract of the HIP kernel.
+    """
+    if negative_slots not in ("reference", "skip"):
+        raise ValueError(negative_slots)
+    kb = _as_bf16_bits(np.asarray(key))          # :70  key.astype(cache.dtype)
+    vb = _as_bf16_bits(np.asarray(value))        # :71
+    slots = np.asarray(slot_mapping, dtype=np.int64)
+    k_new = np.array(k_cache, dtype=np.uint16, copy=True)
+    v_new = np.array(v_cache, dtype=np.uint16, copy=True)
+    num_slots = k_new.shape[0]
+    valid = slots >= 0                           # :64
+    if negative_slots == "reference":
+        safe = np.where(valid, slots, 0)         # :67
+        keep = safe < num_slots                  # mode='drop' (:74)
+    else:
+        safe = slots
+        keep = valid & (slots < num_slots)
+    idx = safe[keep]
+    k_new[idx] = kb[keep]                        # :74
+    v_new[idx] = vb[keep]                        # :75
+    return k_new, v_new
+
+
+# ---------------------------------------------------------------------------
+# Paged decode attention
+# ---------------------------------------------------------------------------
+
+def gather_kv_from_cache_ref(k_cache, v_cache, block_tables, context_lens, block_size):
+    """Restates ``gather_kv_from_cache`` (``layers/attention.py:80-122``):
+    clip tables (:107), gather pages (:111-112), flatten to
+    [B, MB*bs, Hkv, D] (:115-116), mask = pos < ctx (:119-120)."""
+    bt = np.asarray(block_tables)
+    B, MB = bt.shape
+    S = MB * block_size
+    Hkv, D = k_cache.shape[2], k_cache.shape[3]
+    safe = np.clip(bt, 0, k_cache.shape[0] - 1)
+    k = k_cache[safe].reshape(B, S, Hkv, D)
+    v = v_cache[safe].reshape(B, S, Hkv, D)
+    mask = np.arange(S)[None, :] < np.asarray(context_lens)[:, None]
+    return k, v, mask
+
+
+def paged_decode_attention_vectorized_ref(q, k_cache, v_cache, block_tables,
+                                          context_lens, scale, block_size):
+    """Literal restatement of ``paged_decode_attention_vectorized``
+    (``layers/pallas_attention.py:146-238``), whole batch at once.
+
+    q : [B, Hq, D] bf16 bits;  k_cache, v_cache : [NB, bs, Hkv, D] bf16 bits;
+    block_tables : [B, MB] int32 (-1 padded);  context_lens : [B] int32.
+    Returns [B, Hq, D] bf16 bits.
+
+    Materialises [B, MB*bs, Hq, D] fp32 twice, like the reference: use
+    ``paged_decode_attention_per_seq_ref`` for large shapes.
+    """
+    q = np.asarray(q)
+    B, Hq, D = q.shape
+    NB, bs, Hkv, _ = k_cache.shape
+    assert bs == block_size
+    MB = block_tables.shape[1]
+    S = MB * block_size
+    G = Hq // Hkv                                                    # :181
+    safe = np.clip(np.asarray(block_tables), 0, NB - 1)             # :185
+    k_flat = k_cache[safe].reshape(B, S, Hkv, D)                     # :188-192
+    v_flat = v_cache[safe].reshape(B, S, Hkv, D)
+    k_f32 = bf16_bits_to_f32(np.repeat(k_flat, G, axis=2))           # :197, :202
+    v_f32 = bf16_bits_to_f32(np.repeat(v_flat, G, axis=2))           # :198, :203
+    q_f32 = bf16_bits_to_f32(q)                                      # :201
+    scale = np.float32(scale)
+    # scores[b,h,s] = (q[b,h,:] . k[b,s,h,:]) * scale                  :208-214
+    scores = np.einsum("bhd,bshd->bhs", q_f32, k_f32, dtype=np.float32) * scale
+    mask = (np.arange(S)[None, None, :]
+            < np.asarray(context_lens)[:, None, None])               # :216-217
+    scores = np.where(mask, scores, np.float32(-1e9))                # :220
+    smax = scores.max(axis=-1, keepdims=True)                        # :223
+    e = np.exp(scores - smax, dtype=np.float32)                      # :224
+    e = np.where(mask, e, np.float32(0.0))                           # :225
+    ssum = e.sum(axis=-1, keepdims=True, dtype=np.float32)           # :226
+    w = e / (ssum + np.float32(1e-9))                                # :227
+    out = np.einsum("bhs,bshd->bhd", w, v_f32, dtype=np.float32)     # :231-236
+    return f32_to_bf16_bits(out)                                     # :238
+
+
+def paged_decode_attention_per_seq_ref(q, k_cache, v_cache, block_tables,
+                                       context_lens, scale, block_size,
+                                       return_f32: bool = False):
+    """Same arithmetic as ``paged_decode_attention_vectorized_ref``
+    (``layers/pallas_attention.py:146-238``), evaluated one sequence at a time
+    over that sequence's own ceil(ctx/bs) pages so memory stays bounded at the
+    32k-context configs.  Positions >= ctx carry weight exactly 0 in the
+    reference (:225), so restricting to the live pages changes nothing but
+    fp32 summation order.  ctx == 0 gives zeros (0 / (0 + 1e-9), :227).
+    """
+    q = np.asarray(q)
+    B, Hq, D = q.shape
+    NB, bs, Hkv, _ = k_cache.shape
+    assert bs == block_size
+    G = Hq // Hkv
+    bt = np.asarray(block_tables)
+    ctx = np.asarray(context_lens)
+    scale = np.float32(scale)
+    out = np.zeros((B, Hq, D), dtype=np.float32)
+    for b in range(B):
+        n = int(ctx[b])
+        if n <= 0:
+            continue
+        nblk = -(-n // block_size)
+        pages = np.clip(bt[b, :nblk], 0, NB - 1)                     # :185
+        k = bf16_bits_to_f32(k_cache[pages].reshape(nblk * bs, Hkv, D)[:n])
+        v = bf16_bits_to_f32(v_cache[pages].reshape(nblk * bs, Hkv, D)[:n])
+        qb = bf16_bits_to_f32(q[b]).reshape(Hkv, G, D)               # head h -> kv h // G (:197)
+        s = np.einsum("kgd,skd->kgs", qb, k, dtype=np.float32) * scale
+        smax = s.max(axis=-1, keepdims=True)
+        e = np.exp(s - smax, dtype=np.float32)
+        w = e / (e.sum(axis=-1, keepdims=True, dtype=np.float32) + np.float32(1e-9))
+        out[b] = np.einsum("kgs,skd->kgd", w, v, dtype=np.float32).reshape(Hq, D)
+    if return_f32:
+        return out
+    return f32_to_bf16_bits(out)
+
+
+def paged_attention_fallback_ref(q, k_cache, v_cache, block_tables,
+                                 context_lens, scale, block_size):
+    """Restates the gather + ``jax.nn.dot_product_attention`` fallback
+    (``layers/attention.py:399-434``; twin ``_paged_attention_fallback``
+    ``layers/pallas_attention.py:510-550``).
+
+    ``jax.nn.dot_product_attention`` is third-party (jax, not in the reference
+    tree).  Its XLA implementation, as published, computes logits from the
+    bf16 operands with fp32 accumulation, scales, masks, takes the softmax in
+    fp32, casts the probabilities to the value dtype (bf16) and contracts with
+    V with fp32 accumulation, rounding the result to bf16.  GQA maps query
+    head h to kv head h // G.  Fully masked rows (ctx == 0) are not defined by
+    the reference's callers; here they return zeros.
+    """
+    q = np.asarray(q)
+    B, Hq, D = q.shape
+    Hkv = k_cache.shape[2]
+    G = Hq // Hkv
+    kg, vg, mask = gather_kv_from_cache_ref(k_cache, v_cache, block_tables,
+                                            context_lens, block_size)
+    out = np.zeros((B, Hq, D), dtype=np.float32)
+    scale = np.float32(scale)
+    for b in range(B):
+        n = int(mask[b].sum())
+        if n == 0:
+            continue
+        k = bf16_bits_to_f32(kg[b, :n])
+        v = bf16_bits_to_f32(vg[b, :n])
+        qb = bf16_bits_to_f32(q[b]).reshape(Hkv, G, D)
+        s = np.einsum("kgd,skd->kgs", qb, k, dtype=np.float32) * scale
+        s = s - s.max(axis=-1, keepdims=True)
+        e = np.exp(s, dtype=np.float32)
+        p = e / e.sum(axis=-1, keepdims=True, dtype=np.float32)
+        p = bf16_bits_to_f32(f32_to_bf16_bits(p))        # probs.astype(value.dtype)
+        out[b] = np.einsum("kgs,skd->kgd", p, v, dtype=np.float32).reshape(Hq, D)
+    return f32_to_bf16_bits(out)
+
+
+def textbook_attention_f64(q, k_cache, v_cache, block_tables, context_lens,
+                           scale, block_size):
+    """softmax(q K^T * scale) V in float64 with plain Python loops over
+    (sequence, head, position): the independent brute-force statement the
+    restatements above are pinned against on small shapes.  Returns float64
+    [B, Hq, D] (not rounded)."""
+    q = np.asarray(q)
+    B, Hq, D = q.shape
+    NB, bs, Hkv, _ = k_cache.shape
+    G = Hq // Hkv
+    qf = bf16_bits_to_f32(q).astype(np.float64)
+    kf = bf16_bits_to_f32(k_cache).astype(np.float64)
+    vf = bf16_bits_to_f32(v_cache).astype(np.float64)
+    out = np.zeros((B, Hq, D), dtype=np.float64)
+    for b in range(B):
+        n = int(context_lens[b])
+        for h in range(Hq):
+            kvh = h // G
+            logits = np.empty(n, dtype=np.float64)
+            for pos in range(n):
+                page = int(block_tables[b, pos // block_size])
+                logits[pos] = float(scale) * float(qf[b, h] @ kf[page, pos % block_size, kvh])
+            if n == 0:
+                continue
+            w = np.exp(logits - logits.max())
+            w /= w.sum()
+            acc = np.zeros(D, dtype=np.float64)
+            for pos in range(n):
+                page = int(block_tables[b, pos // block_size])
+                acc += w[pos] * vf[page, pos % block_size, kvh]
+            out[b, h] = acc
+    return out

@@ -1,0 +1,133 @@
+"""GPU parity of the HIP paged decode attention against the CPU oracle,
+through the C ABI (via the package's ctypes binding)."""
+import numpy as np
+import pytest
+
+from helpers import ATOL, RTOL, assert_close_bf16, bits_to_torch, make_problem, torch_to_bits
+
+pytestmark = pytest.mark.gpu
+
+
+def run_hip(q, kc, vc, bt, ctx, scale, bs, chunk=0):
+    import torch
+    from nanovllm_jax_amd import paged_attention
+    dev = "cuda:0"
+    out = paged_attention(bits_to_torch(q, dev), bits_to_torch(kc, dev), bits_to_torch(vc, dev),
+                          torch.from_numpy(bt).to(dev), torch.from_numpy(ctx).to(dev),
+                          scale, bs, chunk=chunk)
+    torch.cuda.synchronize()
+    return torch_to_bits(out)
+
+
+def oracle(q, kc, vc, bt, ctx, scale, bs):
+    from oracle.paged_attention_oracle import paged_decode_attention_per_seq_ref
+    return paged_decode_attention_per_seq_ref(q, kc, vc, bt, ctx, scale, bs)
+
+
+@pytest.mark.parametrize("chunk", [0, 32, 64, 256, 1024])
+@pytest.mark.parametrize("Hq,Hkv", [(16, 8), (32, 8), (64, 8), (8, 8), (8, 2), (4, 1)])
+def test_small_random(Hq, Hkv, chunk):
+    print(f"case small_random Hq={Hq} Hkv={Hkv} chunk={chunk}", flush=True)
+    B, D, bs, NB = 5, 128, 64, 40
+    ctx = [1, 31, 64, 97, 300]
+    q, kc, vc, bt, ctx = make_problem(7 + Hq + chunk, B, Hq, Hkv, D, bs, NB, ctx)
+    scale = 1.0 / np.sqrt(D)
+    got = run_hip(q, kc, vc, bt, ctx, scale, bs, chunk)
+    want = oracle(q, kc, vc, bt, ctx, scale, bs)
+    assert_close_bf16(got, want, what=f"Hq={Hq} Hkv={Hkv} chunk={chunk}")
+
+
+def test_c1_shape_vs_vectorized_oracle():
+    """Config C1 (Qwen3-0.6B shape), against the literal whole-batch restatement."""
+    print("case C1", flush=True)
+    from nanovllm_jax_amd.workloads import draw_bf16_bits, make_workload
+    from oracle.paged_attention_oracle import paged_decode_attention_vectorized_ref
+    w = make_workload("C1")
+    rng = np.random.Generator(np.random.PCG64(w.seed + 100))
+    q = draw_bf16_bits(rng, (w.batch, w.num_heads, w.head_dim))
+    kc = draw_bf16_bits(rng, (w.num_blocks, w.block_size, w.num_kv_heads, w.head_dim))
+    vc = draw_bf16_bits(rng, (w.num_blocks, w.block_size, w.num_kv_heads, w.head_dim))
+    got = run_hip(q, kc, vc, w.block_tables, w.context_lens, w.scale, w.block_size)
+    want = paged_decode_attention_vectorized_ref(q, kc, vc, w.block_tables, w.context_lens,
+                                                 w.scale, w.block_size)
+    assert_close_bf16(got, want, what="C1")
+
+
+def test_edge_context_lengths():
+    """ctx = 0 -> zeros; ctx = 1 -> the V row itself, exactly; block boundary
+    and one past it."""
+    print("case edge_context_lengths", flush=True)
+    B, Hq, Hkv, D, bs, NB = 6, 32, 8, 128, 256, 16
+    ctx = [0, 1, 256, 257, 255, 512]
+    q, kc, vc, bt, ctx = make_problem(11, B, Hq, Hkv, D, bs, NB, ctx)
+    scale = 1.0 / np.sqrt(D)
+    got = run_hip(q, kc, vc, bt, ctx, scale, bs)
+    want = oracle(q, kc, vc, bt, ctx, scale, bs)
+    assert_close_bf16(got, want, what="edge")
+    assert not got[0].any(), "ctx=0 must give zeros"
+    G = Hq // Hkv
+    v_first = vc[bt[1, 0], 0]                       # [Hkv, D]
+    assert np.array_equal(got[1], np.repeat(v_first, G, axis=0)), "ctx=1 must return V[0] exactly"
+
+
+def test_padding_and_garbage_are_never_read():
+    """Table entries past the live pages and cache rows past ctx must not
+    matter: poison them (NaN bit patterns / wild page numbers)."""
+    print("case padding_and_garbage", flush=True)
+    B, Hq, Hkv, D, bs, NB = 4, 32, 8, 128, 256, 24
+    ctx = [100, 300, 513, 1000]
+    q, kc, vc, bt, ctx = make_problem(13, B, Hq, Hkv, D, bs, NB, ctx)
+    scale = 1.0 / np.sqrt(D)
+    clean = run_hip(q, kc, vc, bt, ctx, scale, bs)
+    kc2, vc2, bt2 = kc.copy(), vc.copy(), bt.copy()
+    for b in range(B):
+        n = int(ctx[b]); last = (n - 1) // bs
+        page = bt[b, last]
+        kc2[page, n - last * bs:] = 0x7FC0          # NaN
+        vc2[page, n - last * bs:] = 0x7FC0
+        bt2[b, last + 1:] = np.array([2**30, -7, -1, 123456][: bt.shape[1] - last - 1] +
+                                     [-1] * max(0, bt.shape[1] - last - 1 - 4), dtype=np.int32)
+    used = set(int(p) for b in range(B) for p in bt[b, : -(-int(ctx[b]) // bs)])
+    for p in range(NB):
+        if p not in used:
+            kc2[p] = 0x7FC0; vc2[p] = 0x7FC0
+    dirty = run_hip(q, kc2, vc2, bt2, ctx, scale, bs)
+    assert np.array_equal(clean, dirty)
+
+
+def test_split_invariance_and_page_permutation():
+    print("case split_invariance", flush=True)
+    from oracle.paged_attention_oracle import bf16_bits_to_f32
+    B, Hq, Hkv, D, bs, NB = 3, 32, 8, 128, 256, 20
+    ctx = [1500, 777, 2048]
+    q, kc, vc, bt, ctx = make_problem(17, B, Hq, Hkv, D, bs, NB, ctx)
+    scale = 1.0 / np.sqrt(D)
+    outs = [bf16_bits_to_f32(run_hip(q, kc, vc, bt, ctx, scale, bs, ch)) for ch in (32, 128, 256, 2048)]
+    for o in outs[1:]:
+        np.testing.assert_allclose(o, outs[0], atol=ATOL, rtol=RTOL)
+    # move every page somewhere else: same logical content, other physical layout
+    perm = np.random.Generator(np.random.PCG64(5)).permutation(NB)
+    kc2 = np.empty_like(kc); vc2 = np.empty_like(vc)
+    kc2[perm] = kc; vc2[perm] = vc
+    bt2 = np.where(bt >= 0, perm[np.clip(bt, 0, NB - 1)], -1).astype(np.int32)
+    moved = run_hip(q, kc2, vc2, bt2, ctx, scale, bs, 256)
+    assert np.array_equal(moved, run_hip(q, kc, vc, bt, ctx, scale, bs, 256))
+
+
+def test_reference_smoke_shape_b64():
+    """Shape of the reference's decode smoke test (test_mosaic_kernels.py:30-54):
+    B=64, Hq=32, Hkv=8, D=128, 128 pages of 256, tables arange % 128,
+    ctx = min(200 + 50 i, 2048)."""
+    print("case reference_smoke_b64", flush=True)
+    from nanovllm_jax_amd.workloads import draw_bf16_bits
+    B, Hq, Hkv, D, bs, NB, MB = 64, 32, 8, 128, 256, 128, 8
+    rng = np.random.Generator(np.random.PCG64(42))
+    q = draw_bf16_bits(rng, (B, Hq, D))
+    kc = draw_bf16_bits(rng, (NB, bs, Hkv, D))
+    vc = draw_bf16_bits(rng, (NB, bs, Hkv, D))
+    bt = (np.arange(B * MB, dtype=np.int32).reshape(B, MB) % NB).astype(np.int32)
+    ctx = np.minimum(200 + 50 * np.arange(B), 2048).astype(np.int32)
+    scale = 1.0 / np.sqrt(D)
+    got = run_hip(q, kc, vc, bt, ctx, scale, bs)
+    want = oracle(q, kc, vc, bt, ctx, scale, bs)
+    assert_close_bf16(got, want, what="reference smoke shape")
