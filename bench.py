@@ -77,29 +77,46 @@ def timed(fn, steps, torch):
 
 
 def cpu_baseline(w, q, kc, vc, budget_s=20.0):
-    """Oracle on the host cores over the first sequences of the batch until
-    the time budget is used; extrapolated linearly in live positions."""
-    from oracle.paged_attention_oracle import paged_decode_attention_per_seq_ref
+    """The CPU oracle on the host cores (C restatement, OpenMP over
+    (sequence, kv head)), same inputs, on a bounded sample: whole calls over
+    the first `n` sequences of the batch, 2 warm-up + up to 5 timed calls
+    within the time budget; median.  Falls back to the single-threaded NumPy
+    restatement when the C oracle has not been built."""
     from nanovllm_jax_amd.workloads import algorithmic_bytes
+    from oracle import c_oracle
     qb, kb, vb = to_bits(q), to_bits(kc), to_bits(vc)
-    done_pos, done_seq, t_used = 0, 0, 0.0
-    b = 0
-    while b < w.batch and t_used < budget_s:
-        n = min(4, w.batch - b)
+    if c_oracle.available():
+        fn, cores, impl = c_oracle.paged_decode, c_oracle.num_threads(), "C oracle (OpenMP)"
+    else:
+        from oracle.paged_attention_oracle import paged_decode_attention_per_seq_ref
+        fn, cores, impl = paged_decode_attention_per_seq_ref, 1, "NumPy oracle"
+
+    def call(n):
         t0 = time.perf_counter()
-        paged_decode_attention_per_seq_ref(qb[b:b + n], kb, vb, w.block_tables[b:b + n],
-                                           w.context_lens[b:b + n], w.scale, w.block_size)
-        t_used += time.perf_counter() - t0
-        done_pos += int(w.context_lens[b:b + n].sum())
-        done_seq += n
-        b += n
-    byts = algorithmic_bytes(w.context_lens[:done_seq], done_seq, w.num_heads, w.num_kv_heads,
-                             w.head_dim, w.max_blocks)
-    return {"value": round(byts / t_used / 1e9, 4), "unit": "GB/s", "cores": 1, "kind": "port",
-            "us_per_call_extrapolated": round(
-                t_used / max(done_pos, 1) * int(w.context_lens.sum()) * 1e6, 1),
-            "sample": f"NumPy oracle (single thread) on the first {done_seq} of {w.batch} "
-                      f"sequences of {w.name} ({done_pos} positions, {t_used:.1f} s)"}
+        fn(qb[:n], kb, vb, w.block_tables[:n], w.context_lens[:n], w.scale, w.block_size)
+        return time.perf_counter() - t0
+
+    # size the sample so one call costs at most ~1/7 of the budget
+    n = min(w.batch, max(1, cores))
+    t = call(n)
+    while n < w.batch and t * 2 < budget_s / 7:
+        n = min(w.batch, n * 2)
+        t = call(n)
+    times = []
+    spent = 0.0
+    call(n)
+    while len(times) < 5 and (spent + t < budget_s or not times):
+        t = call(n)
+        times.append(t)
+        spent += t
+    med = float(np.median(times))
+    byts = algorithmic_bytes(w.context_lens[:n], n, w.num_heads, w.num_kv_heads, w.head_dim,
+                             w.max_blocks)
+    pos = int(w.context_lens[:n].sum())
+    return {"value": round(byts / med / 1e9, 3), "unit": "GB/s", "cores": cores, "kind": "port",
+            "us_per_call_full_batch": round(med / max(pos, 1) * int(w.context_lens.sum()) * 1e6, 1),
+            "sample": f"{impl}, {cores} threads, first {n} of {w.batch} sequences of {w.name} "
+                      f"({pos} positions), median of {len(times)} calls of {med * 1e3:.1f} ms"}
 
 
 def main():
@@ -110,6 +127,9 @@ def main():
     ap.add_argument("--workload", default="C2", choices=["C1", "C2", "C3", "C4", "C5"])
     ap.add_argument("--chunk", type=int, default=0, help="positions per workgroup (0 = default)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--copy-calibration", action="store_true",
+                    help="also run a plain 1 GiB device-to-device copy a few times, so a "
+                         "counter run has a kernel of known traffic to scale against")
     ap.add_argument("--cpu-budget", type=float, default=20.0)
     args = ap.parse_args()
     if args.gpus != 1:
@@ -145,6 +165,14 @@ def main():
 
     def store():
         store_kv_to_cache(k_new, v_new, kflat, vflat, slots)
+
+    if args.copy_calibration:
+        src = torch.empty(1 << 30, dtype=torch.uint8, device=dev).fill_(1)
+        dst = torch.empty_like(src)
+        for _ in range(5):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
 
     store()
     for _ in range(args.warmup):

@@ -332,13 +332,14 @@ int round_up(int x, int m) { return (x + m - 1) / m * m; }
 extern "C" int32_t nvj_paged_decode_default_chunk(int32_t batch, int32_t num_kv_heads,
                                                   int32_t max_blocks, int32_t block_size) {
   if (batch <= 0 || num_kv_heads <= 0 || max_blocks <= 0 || block_size <= 0) return 256;
-  // Aim for a few thousand workgroups when every sequence is full length
-  // (256 CUs, one or two resident workgroups each), never below 64 positions
-  // and never above one 256-position page.
+  // One workgroup (8 waves at ~230 VGPRs) is resident per CU, so with every
+  // sequence at full length the launch should be about one workgroup per CU
+  // (256 on MI355X).  Longer chunks than 1024 positions leave ragged batches
+  // badly balanced; shorter ones than 128 only add partials to combine.
   const int64_t positions = (int64_t)batch * max_blocks * block_size;
-  int64_t chunk = positions / 2048;
-  if (chunk < 64) chunk = 64;
-  if (chunk > 256) chunk = 256;
+  int64_t chunk = (positions + 255) / 256;
+  if (chunk < 128) chunk = 128;
+  if (chunk > 1024) chunk = 1024;
   return round_up((int)chunk, kStep);
 }
 

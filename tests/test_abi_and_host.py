@@ -1,0 +1,145 @@
+"""CPU-side checks: the C-ABI library loads and exports every symbol the header
+declares; the host mirror validates its arguments and never computes on the
+CPU; workload metadata follows the reference's filler formulas."""
+import ctypes
+import os
+import re
+
+import numpy as np
+import pytest
+import torch
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def header_symbols():
+    text = open(os.path.join(ROOT, "include", "nvj_paged_attn.h")).read()
+    return re.findall(r"NVJ_API\s+[\w\s\*]+?\b(nvj_\w+)\s*\(", text)
+
+
+def test_library_exports_every_declared_symbol():
+    from nanovllm_jax_amd import _lib
+    names = header_symbols()
+    assert len(names) >= 7 and len(set(names)) == len(names)
+    raw = ctypes.CDLL(_lib.lib_path())
+    for n in names:
+        assert hasattr(raw, n), f"{n} declared in the header but not exported"
+    assert set(names) == set(_lib.SYMBOLS), "ctypes table and header disagree"
+    lib = _lib.load()
+    assert lib.nvj_abi_version() == _lib.NVJ_ABI_VERSION
+    assert lib.nvj_error_string(0) == b"ok"
+    for code in range(-6, 0):
+        assert lib.nvj_error_string(code) not in (b"ok", b"unknown error code")
+
+
+def test_argument_validation_without_a_gpu():
+    """Entry points reject bad arguments before touching the device."""
+    from nanovllm_jax_amd import _lib
+    lib = _lib.load()
+    L = lib.nvj_paged_decode_launch
+    ok = dict(batch=2, Hq=32, Hkv=8, D=128, bs=256, MB=4, NB=16)
+
+    def call(**kw):
+        a = dict(ok); a.update(kw)
+        p = kw.get("ptr", 0x1000)
+        return L(None, p, p, p, p, p, p, p, 1 << 30, a["batch"], a["Hq"], a["Hkv"], a["D"],
+                 a["bs"], a["MB"], a["NB"], 0.1, kw.get("chunk", 0))
+
+    assert call(D=64) == -3                # head_dim not built
+    assert call(Hq=30) == -2               # Hq % Hkv
+    assert call(Hq=256, Hkv=8) == -3       # group > 16
+    assert call(bs=48) == -3
+    assert call(chunk=100) == -3
+    assert call(batch=-1) == -2
+    assert call(batch=0) == 0              # empty batch: nothing to do
+    assert call(ptr=0) == -1
+    assert call(ptr=0x1004) == -4          # misaligned
+    assert L(None, 0x1000, 0x1000, 0x1000, 0x1000, 0x1000, 0x1000, 0x1000, 16, 2, 32, 8, 128, 256,
+             4, 16, 0.1, 0) == -4          # workspace too small
+    S = lib.nvj_store_kvcache_launch
+    assert S(None, 0, 0, 0, 0, 0, 0, 8, 128, 1024, 0, 0) == 0       # no tokens
+    assert S(None, 0x1000, 0x1000, 0x1000, 0x1000, 0x1000, 4, 8, 128, 1024, 7, 0) == -6
+    assert S(None, 0, 0x1000, 0x1000, 0x1000, 0x1000, 4, 8, 128, 1024, 0, 0) == -1
+    assert S(None, 0x1000, 0x1000, 0x1000, 0x1000, 0x1000, 4, 3, 3, 1024, 0, 0) == -3
+    assert S(None, 0x1000, 0x1000, 0x1000, 0x1000, 0x1000, -4, 8, 128, 1024, 0, 0) == -2
+
+
+def test_workspace_and_chunk_queries():
+    from nanovllm_jax_amd.layers.paged_attention import default_chunk, paged_decode_workspace_bytes
+    c = default_chunk(64, 8, 16, 256)
+    assert c % 32 == 0 and 32 <= c <= 4096
+    need = paged_decode_workspace_bytes(64, 32, 128, 16, 256, 8, 256)
+    assert need == 64 * 16 * 32 * (128 + 2) * 4
+    assert paged_decode_workspace_bytes(64, 32, 128, 16, 256, 8, 100) == 0   # bad chunk
+    assert paged_decode_workspace_bytes(64, 32, 128, 16, 256, 8, 0) == \
+        paged_decode_workspace_bytes(64, 32, 128, 16, 256, 8, c)
+
+
+def test_host_mirror_refuses_cpu_tensors():
+    """No CPU fallback: host tensors are an error, not a slow path."""
+    from nanovllm_jax_amd import Attention, create_decode_context, paged_attention, store_kv_to_cache
+    q = torch.zeros(2, 32, 128, dtype=torch.bfloat16)
+    kc = torch.zeros(4, 256, 8, 128, dtype=torch.bfloat16)
+    bt = torch.zeros(2, 2, dtype=torch.int32)
+    ctx = torch.ones(2, dtype=torch.int32)
+    with pytest.raises(ValueError, match="GPU"):
+        paged_attention(q, kc, kc.clone(), bt, ctx, 0.1, 256)
+    with pytest.raises(ValueError, match="GPU"):
+        store_kv_to_cache(torch.zeros(2, 8, 128), torch.zeros(2, 8, 128), kc.view(-1, 8, 128),
+                          kc.view(-1, 8, 128).clone(), torch.zeros(2, dtype=torch.int32))
+    attn = Attention(32, 128, 0.1, 8, 256)
+    c = create_decode_context(ctx, torch.zeros(2, dtype=torch.int32), bt)
+    assert c.is_prefill is False and c.last_token_indices is None
+    with pytest.raises(RuntimeError, match="set_kv_cache"):
+        attn(q, q, q, c)
+    attn.set_kv_cache(kc, kc.clone())
+    c.is_prefill = True
+    with pytest.raises(NotImplementedError):
+        attn(q, q, q, c)
+
+
+def test_missing_library_fails_loudly(monkeypatch, tmp_path):
+    from nanovllm_jax_amd import _lib
+    monkeypatch.setattr(_lib, "_lib", None)
+    monkeypatch.setattr(_lib, "_LIB_PATH", str(tmp_path / "nope.so"))
+    with pytest.raises(_lib.NativeLibraryError, match="no fallback"):
+        _lib.load()
+
+
+def test_product_never_imports_the_oracle():
+    pkg = os.path.join(ROOT, "nanovllm_jax_amd")
+    for dirpath, _, files in os.walk(pkg):
+        for f in files:
+            if f.endswith((".py", ".hip", ".h", ".cc")):
+                text = open(os.path.join(dirpath, f)).read()
+                assert not re.search(r"^\s*(from|import)\s+oracle\b", text, re.M), f
+                assert "paged_oracle" not in text, f
+
+
+@pytest.mark.parametrize("name", ["C1", "C2", "C3", "C4", "C5"])
+def test_workload_metadata(name):
+    from nanovllm_jax_amd.workloads import algorithmic_bytes, make_workload
+    w = make_workload(name)
+    bs = w.block_size
+    assert w.block_tables.shape == (w.batch, w.max_blocks) and w.block_tables.dtype == np.int32
+    nblk = -(-w.context_lens // bs)
+    live = np.arange(w.max_blocks)[None, :] < nblk[:, None]
+    assert (w.block_tables[~live] == -1).all()                       # -1 padding
+    pages = w.block_tables[live]
+    assert pages.min() >= 0 and pages.max() < w.num_blocks and len(set(pages.tolist())) == len(pages)
+    # slot = block_table[-1] * block_size + last_block_num_tokens - 1
+    for b in range(0, w.batch, max(1, w.batch // 8)):
+        n = int(w.context_lens[b])
+        last_tokens = n - (nblk[b] - 1) * bs
+        assert w.slot_mapping[b] == w.block_tables[b, nblk[b] - 1] * bs + last_tokens - 1
+    same = make_workload(name)
+    assert np.array_equal(same.block_tables, w.block_tables)          # seeded
+    if name == "C2":
+        assert algorithmic_bytes(w.context_lens, w.batch, w.num_heads, w.num_kv_heads,
+                                 w.head_dim, w.max_blocks) == 1_074_794_752
+    if name == "C4":
+        assert algorithmic_bytes(w.context_lens, w.batch, w.num_heads, w.num_kv_heads,
+                                 w.head_dim, w.max_blocks) == 2_148_016_192
+    if name == "C3":
+        assert w.context_lens.min() >= 16 and w.context_lens.max() <= 32768
+        assert w.num_blocks == int(np.ceil(1.1 * nblk.sum()))
