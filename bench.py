@@ -133,8 +133,9 @@ def main():
     ap.add_argument("--cpu-budget", type=float, default=20.0)
     args = ap.parse_args()
     if args.gpus != 1:
-        print("bench.py: this build runs on ONE GPU only (the path shards with no exchange "
-              "step; see DESIGN.md); --gpus must be 1", file=sys.stderr)
+        print("bench.py: this build runs on ONE GPU only (every (sequence, kv head) pair is "
+              "independent, so more GPUs would just split the batch); --gpus must be 1",
+              file=sys.stderr)
         return 2
 
     import torch
