@@ -67,8 +67,12 @@ __device__ __forceinline__ uint32_t slot_offset(int x, int last, uint32_t row_by
   return (uint32_t)x * row_bytes + lane_bytes;
 }
 
+// K/V are read exactly once per call: non-temporal loads stream them past the
+// caches instead of allocating lines that will never be hit again.
 __device__ __forceinline__ uint4 load_piece(const char* base, uint32_t off) {
-  return *reinterpret_cast<const uint4*>(base + off);
+  typedef __attribute__((ext_vector_type(4))) unsigned int u32x4;
+  const u32x4 t = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(base + off));
+  return make_uint4(t[0], t[1], t[2], t[3]);
 }
 
 // K of one step: load slot i of lane (kg, r) is position 4*i + kg, piece r, so
@@ -332,14 +336,17 @@ int round_up(int x, int m) { return (x + m - 1) / m * m; }
 extern "C" int32_t nvj_paged_decode_default_chunk(int32_t batch, int32_t num_kv_heads,
                                                   int32_t max_blocks, int32_t block_size) {
   if (batch <= 0 || num_kv_heads <= 0 || max_blocks <= 0 || block_size <= 0) return 256;
-  // One workgroup (8 waves at ~230 VGPRs) is resident per CU, so with every
-  // sequence at full length the launch should be about one workgroup per CU
-  // (256 on MI355X).  Longer chunks than 1024 positions leave ragged batches
-  // badly balanced; shorter ones than 128 only add partials to combine.
+  // One workgroup (8 waves at ~230 VGPRs) is resident per CU, and the kernel
+  // is fastest when a launch is exactly one workgroup per CU (256 on MI355X):
+  // pick the chunk that gives that when every sequence is at full length, if
+  // it is at most 2048 positions.  Beyond that the launch runs in several
+  // rounds anyway and 1024 keeps ragged batches balanced (a long chunk that
+  // starts late becomes the tail of the whole launch).  Below 128 positions
+  // the partials only add combine work.
   const int64_t positions = (int64_t)batch * max_blocks * block_size;
   int64_t chunk = (positions + 255) / 256;
   if (chunk < 128) chunk = 128;
-  if (chunk > 1024) chunk = 1024;
+  if (chunk > 2048) chunk = 1024;
   return round_up((int)chunk, kStep);
 }
 
