@@ -125,6 +125,39 @@ def cpu_baseline(w, q, kc, vc, budget_s=20.0):
                       f"({pos} positions), median of {len(times)} calls of {med * 1e3:.1f} ms"}
 
 
+def bench_decode_step(args, torch):
+    """Whole-model decode step at the Qwen3-0.6B shape: 28 layers, B=128, every
+    sequence at context 1024, page 256, random bf16 weights, greedy pick; the
+    step is one HIP graph.  Reports decode tokens/s."""
+    from nanovllm_jax_amd.engine.decode_step import DecodeModelConfig, DecodeStepRunner
+    cfg = DecodeModelConfig()
+    batch, ctx_len = 128, 1024
+    runner = DecodeStepRunner(cfg, "cuda:0", seed=1005)
+    rng = np.random.Generator(np.random.PCG64(1005))
+    pages = rng.permutation(cfg.num_kvcache_blocks).reshape(batch, -1)[:, :ctx_len // cfg.block_size]
+    last = rng.integers(0, cfg.vocab_size, batch).tolist()
+    ids, pos, ctx = runner.make_inputs(last, [ctx_len] * batch, pages.tolist())
+    eager = runner.step(ids, pos, ctx).clone()
+    replay = runner.capture(ids, pos, ctx)
+    same = bool(torch.equal(replay(), eager))
+    for _ in range(args.warmup):
+        replay()
+    ms, wall = timed(replay, args.steps, torch)
+    ms_eager, _ = timed(lambda: runner.step(ids, pos, ctx), max(3, args.steps // 10), torch)
+    kv_bytes = cfg.num_layers * batch * ctx_len * cfg.num_kv_heads * cfg.head_dim * 2 * 2
+    rec = {"metric": "decode tokens/s, Qwen3-0.6B shape whole-model decode step", "value":
+           round(batch / (ms * 1e-3), 1), "unit": "tokens/s", "n_gpus": 1, "steps": args.steps,
+           "warmup": args.warmup, "ms_per_step": round(wall, 4), "higher_is_better": True,
+           "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
+           "config": {"workload": "C5: 28 layers, hidden 1024, Hq=16, Hkv=8, D=128, vocab 151936, "
+                                  "B=128, ctx=1024, page=256, random-init weights, greedy",
+                      "step": "one HIP graph: embedding .. LM head .. argmax",
+                      "kv_bytes_per_step": kv_bytes},
+           "ms_per_step_eager": round(ms_eager, 4), "graph_matches_eager": same}
+    print(json.dumps(rec), flush=True)
+    return 0
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -137,6 +170,9 @@ def main():
                     help="also run a plain 1 GiB device-to-device copy a few times, so a "
                          "counter run has a kernel of known traffic to scale against")
     ap.add_argument("--cpu-budget", type=float, default=20.0)
+    ap.add_argument("--decode-step", action="store_true",
+                    help="time the whole-model decode step (config C5) instead of the "
+                         "attention call; prints its own JSON line")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on ONE GPU only (every (sequence, kv head) pair is "
@@ -156,6 +192,8 @@ def main():
 
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
+    if args.decode_step:
+        return bench_decode_step(args, torch)
     w = make_workload(args.workload)
     q, kc, vc, bt, ctx, slots, k_new, v_new = device_inputs(w, torch, dev)
     chunk = args.chunk or default_chunk(w.batch, w.num_kv_heads, w.max_blocks, w.block_size)

@@ -1,0 +1,214 @@
+"""Whole-model decode step harness around the HIP attention path.
+
+The measured path of this package is the KV-cache store and the paged decode
+attention; everything else a decode step needs (embedding, RMSNorm, the QKV /
+output / MLP projections, RoPE, the LM head, greedy pick) is plain
+``torch`` here (hipBLASLt GEMMs), written from the architecture the reference
+describes: ``models/qwen3.py:130-172`` (attention block: fused QKV, per-head
+QK-RMSNorm when there is no QKV bias, RoPE, attention, output projection),
+``:285-318`` (pre-norm decoder layer with fused residual), ``:366-393`` (stack
++ final norm), ``:472-491`` (tied LM head), ``layers/layernorm.py:31-79``,
+``layers/rotary_embedding.py:13-37,50-106``, ``layers/activation.py:22-33``.
+Cache allocation, wiring and the per-step metadata follow
+``engine/model_runner.py:140-204, 225-246, 334-376``.
+
+Weights are random (N(0, 0.02), bf16); greedy = argmax of the logits, the
+temperature -> 0 limit of the reference's Gumbel-max sampler
+(``layers/sampler.py:39-48``).
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass
+
+import numpy as np
+import torch
+import torch.nn.functional as F
+
+from ..layers.attention import Attention
+from ..layers.paged_attention import paged_decode_workspace_bytes
+from ..utils.context import AttentionContext, create_decode_context
+
+__all__ = ["DecodeModelConfig", "DecodeStepRunner", "prepare_block_tables", "prepare_decode"]
+
+
+@dataclass
+class DecodeModelConfig:
+    """Qwen3-0.6B shape by default."""
+    num_layers: int = 28
+    hidden_size: int = 1024
+    num_heads: int = 16
+    num_kv_heads: int = 8
+    head_dim: int = 128
+    intermediate_size: int = 3072
+    vocab_size: int = 151936
+    rms_norm_eps: float = 1e-6
+    rope_theta: float = 1e6
+    max_position: int = 4096
+    block_size: int = 256
+    num_kvcache_blocks: int = 512
+
+
+def prepare_block_tables(block_tables: list[list[int]]) -> np.ndarray:
+    """Rows padded with -1 to the longest table (``engine/model_runner.py:225-246``)."""
+    width = max(len(t) for t in block_tables)
+    out = np.full((len(block_tables), width), -1, dtype=np.int32)
+    for i, t in enumerate(block_tables):
+        out[i, :len(t)] = t
+    return out
+
+
+def prepare_decode(last_tokens, seq_lens, block_tables, block_size):
+    """Host filler of one decode step (``engine/model_runner.py:334-376``):
+    ``positions = len - 1``, ``context_lens = len``,
+    ``slot = block_table[-1] * block_size + last_block_num_tokens - 1``."""
+    n = len(seq_lens)
+    input_ids = np.asarray(last_tokens, dtype=np.int32)
+    positions = np.empty(n, np.int32)
+    context_lens = np.empty(n, np.int32)
+    slot_mapping = np.empty(n, np.int32)
+    for i, (length, table) in enumerate(zip(seq_lens, block_tables)):
+        positions[i] = length - 1
+        context_lens[i] = length
+        last_block_tokens = length - (len(table) - 1) * block_size
+        slot_mapping[i] = table[-1] * block_size + last_block_tokens - 1
+    return input_ids, positions, context_lens, slot_mapping, prepare_block_tables(block_tables)
+
+
+class DecodeStepRunner:
+    """Owns random weights, the KV cache ``[2, L, NB, bs, Hkv, D]`` bf16 and one
+    ``Attention`` per layer; ``step`` runs one decode step for a batch."""
+
+    def __init__(self, cfg: DecodeModelConfig, device="cuda:0", seed: int = 0,
+                 fill_cache: bool = True):
+        self.cfg = cfg
+        self.device = torch.device(device)
+        g = torch.Generator(device=self.device)
+        g.manual_seed(seed)
+        c = cfg
+
+        def w(*shape):
+            return (torch.randn(shape, generator=g, device=self.device, dtype=torch.float32)
+                    * 0.02).to(torch.bfloat16)
+
+        qkv_out = (c.num_heads + 2 * c.num_kv_heads) * c.head_dim
+        self.embed = w(c.vocab_size, c.hidden_size)            # tied with the LM head
+        self.layers = []
+        for _ in range(c.num_layers):
+            self.layers.append(dict(
+                ln1=torch.ones(c.hidden_size, device=self.device),
+                ln2=torch.ones(c.hidden_size, device=self.device),
+                qkv=w(qkv_out, c.hidden_size),
+                o=w(c.hidden_size, c.num_heads * c.head_dim),
+                q_norm=torch.ones(c.head_dim, device=self.device),
+                k_norm=torch.ones(c.head_dim, device=self.device),
+                gate_up=w(2 * c.intermediate_size, c.hidden_size),
+                down=w(c.hidden_size, c.intermediate_size)))
+        self.final_norm = torch.ones(c.hidden_size, device=self.device)
+        inv_freq = 1.0 / (c.rope_theta ** (torch.arange(0, c.head_dim, 2, dtype=torch.float32,
+                                                        device=self.device) / c.head_dim))
+        freqs = torch.outer(torch.arange(c.max_position, dtype=torch.float32,
+                                         device=self.device), inv_freq)
+        self.cos_sin = torch.cat([freqs.cos(), freqs.sin()], dim=-1)     # [max_pos, D] f32
+        # KV cache, engine/model_runner.py:176,190
+        shape = (2, c.num_layers, c.num_kvcache_blocks, c.block_size, c.num_kv_heads, c.head_dim)
+        self.kv_cache = torch.zeros(shape, dtype=torch.bfloat16, device=self.device)
+        if fill_cache:
+            for layer in range(c.num_layers):
+                for kv in range(2):
+                    self.kv_cache[kv, layer] = torch.randn(
+                        shape[2:], generator=g, device=self.device,
+                        dtype=torch.float32).to(torch.bfloat16)
+        self.attn = []
+        for layer in range(c.num_layers):                        # _wire_kv_cache, :195-204
+            a = Attention(c.num_heads, c.head_dim, c.head_dim ** -0.5, c.num_kv_heads,
+                          c.block_size)
+            a.set_kv_cache(self.kv_cache[0, layer], self.kv_cache[1, layer])
+            self.attn.append(a)
+        self._graph = None
+
+    # -- small torch pieces -------------------------------------------------
+    def _rms(self, x, weight, residual=None):
+        """RMSNorm, optionally fused with the residual add (layernorm.py:31-79)."""
+        if residual is not None:
+            xf = x.float() + residual.float()
+            residual = xf.to(x.dtype)
+        else:
+            xf = x.float()
+            residual = x
+        var = xf.pow(2).mean(-1, keepdim=True)
+        return (xf * torch.rsqrt(var + self.cfg.rms_norm_eps) * weight).to(x.dtype), residual
+
+    def _rope(self, x, cos, sin):
+        """x bf16 [T, H, D]; result float32 like the reference's promotion
+        (rotary_embedding.py:31-37)."""
+        x1, x2 = x.chunk(2, dim=-1)
+        return torch.cat([x1 * cos - x2 * sin, x2 * cos + x1 * sin], dim=-1)
+
+    def forward(self, input_ids, positions, context: AttentionContext):
+        c = self.cfg
+        h = F.embedding(input_ids.long(), self.embed)
+        residual = None
+        cs = self.cos_sin[positions.long()][:, None, :]
+        cos, sin = cs.chunk(2, dim=-1)
+        qs, ks = c.num_heads * c.head_dim, c.num_kv_heads * c.head_dim
+        for lw, attn in zip(self.layers, self.attn):
+            if residual is None:
+                h, residual = self._rms(h, lw["ln1"])
+            else:
+                h, residual = self._rms(h, lw["ln1"], residual)
+            qkv = F.linear(h, lw["qkv"])
+            q, k, v = qkv.split([qs, ks, ks], dim=-1)
+            q = q.reshape(-1, c.num_heads, c.head_dim)
+            k = k.reshape(-1, c.num_kv_heads, c.head_dim)
+            v = v.reshape(-1, c.num_kv_heads, c.head_dim).contiguous()
+            q, _ = self._rms(q, lw["q_norm"])
+            k, _ = self._rms(k, lw["k_norm"])
+            q = self._rope(q, cos, sin)                 # f32
+            k = self._rope(k, cos, sin).contiguous()    # f32, the store rounds it to bf16
+            o = attn(q.to(torch.bfloat16).contiguous(), k, v, context)
+            h = F.linear(o.reshape(-1, qs), lw["o"])
+            h, residual = self._rms(h, lw["ln2"], residual)
+            gate, up = F.linear(h, lw["gate_up"]).chunk(2, dim=-1)
+            h = F.linear(F.silu(gate) * up, lw["down"])
+        h, _ = self._rms(h, self.final_norm, residual)
+        return F.linear(h, self.embed)                   # logits [T, vocab]
+
+    # -- one decode step ------------------------------------------------------
+    def make_inputs(self, last_tokens, seq_lens, block_tables):
+        ids, pos, ctx, slots, bt = prepare_decode(last_tokens, seq_lens, block_tables,
+                                                  self.cfg.block_size)
+        d = self.device
+        t = lambda a: torch.from_numpy(a).to(d)
+        return t(ids), t(pos), create_decode_context(t(ctx), t(slots), t(bt))
+
+    def step(self, input_ids, positions, context):
+        """Eager decode step: logits -> greedy token ids [batch] int64."""
+        return self.forward(input_ids, positions, context).argmax(dim=-1)
+
+    def capture(self, input_ids, positions, context):
+        """Capture the whole step in one HIP graph over static input buffers;
+        returns ``replay() -> token ids`` (the inputs may be updated in place
+        between replays)."""
+        c = self.cfg
+        batch, max_blocks = context.block_tables.shape
+        ws = torch.empty(paged_decode_workspace_bytes(batch, c.num_heads, c.head_dim, max_blocks,
+                                                      c.block_size, c.num_kv_heads, 0),
+                         dtype=torch.uint8, device=self.device)
+        for a in self.attn:
+            a.workspace = ws
+        s = torch.cuda.Stream(self.device)
+        s.wait_stream(torch.cuda.current_stream(self.device))
+        with torch.cuda.stream(s):
+            for _ in range(2):
+                self.step(input_ids, positions, context)
+        torch.cuda.current_stream(self.device).wait_stream(s)
+        torch.cuda.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            out = self.step(input_ids, positions, context)
+        self._graph = graph
+
+        def replay():
+            graph.replay()
+            return out
+        return replay

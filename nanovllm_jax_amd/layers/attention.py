@@ -95,6 +95,9 @@ class Attention:
         self.block_size = block_size
         self.k_cache = None
         self.v_cache = None
+        # optional caller-owned split-K workspace (uint8 device tensor) shared by
+        # the calls of one stream; None = a fresh one per call
+        self.workspace = None
 
     def set_kv_cache(self, k_cache, v_cache):
         self.k_cache = k_cache
@@ -103,7 +106,8 @@ class Attention:
     def _decode_attention(self, q, context: AttentionContext):
         q = q.to(self.k_cache.dtype)      # layers/attention.py:386-387
         return paged_attention(q, self.k_cache, self.v_cache, context.block_tables,
-                               context.context_lens, self.scale, self.block_size)
+                               context.context_lens, self.scale, self.block_size,
+                               workspace=self.workspace)
 
     def __call__(self, q, k, v, context: AttentionContext):
         if self.k_cache is None or self.v_cache is None:
