@@ -146,6 +146,43 @@ NVJ_API int nvj_paged_decode_launch_phases(void* stream,
                             int32_t num_blocks, float scale, int32_t chunk,
                             uint32_t phases);
 
+/*
+ * Fused per-head QK-RMSNorm + rotary embedding + KV-cache store: everything the
+ * reference runs between the QKV projection and the attention call, in one
+ * launch.  Replaces q_norm / k_norm (models/qwen3.py:157-160,
+ * layers/layernorm.py:31-48), rotary_emb (models/qwen3.py:163,
+ * layers/rotary_embedding.py:13-37, 96-106), the cast of q to the cache dtype
+ * (layers/attention.py:386-387) and store_kv_to_cache (layers/attention.py:42-77).
+ *
+ *   qkv            [num_tokens, qkv_row_stride] bf16: per token the
+ *                  num_heads q heads, then num_kv_heads k heads, then
+ *                  num_kv_heads v heads, head_dim each (the fused projection
+ *                  output, models/qwen3.py:147-155); qkv_row_stride in elements
+ *   positions      [num_tokens] int32, clamped into [0, max_position)
+ *   cos_sin_cache  [max_position, head_dim] f32: cos of the head_dim/2
+ *                  frequencies, then sin (layers/rotary_embedding.py:60-76)
+ *   q_norm_weight, k_norm_weight  [head_dim] f32, or both NULL for no QK norm
+ *                  (the reference norms only when there is no QKV bias,
+ *                  models/qwen3.py:125-131)
+ *   slot_mapping   [num_tokens] int32; < 0 skips the token's K/V, >= num_slots
+ *                  drops it (q_out is written for every token)
+ *   k_cache, v_cache [num_slots, num_kv_heads, head_dim] bf16, updated in place
+ *   q_out          [num_tokens, num_heads, head_dim] bf16
+ *
+ * Arithmetic: the fixed IEEE fp32 sequence documented at the top of
+ * csrc/qk_norm_rope_store.hip (xor-butterfly sum of squares, exact 1/sqrt,
+ * normalised value rounded to bf16 before the rotation, rotation in fp32,
+ * result rounded to nearest-even bf16).  head_dim must be 128.
+ */
+NVJ_API int nvj_qk_norm_rope_store_launch(void* stream,
+                            const void* qkv, int64_t qkv_row_stride,
+                            const int32_t* positions, const float* cos_sin_cache,
+                            int32_t max_position, const float* q_norm_weight,
+                            const float* k_norm_weight, float eps,
+                            const int32_t* slot_mapping, void* k_cache, void* v_cache,
+                            void* q_out, int32_t num_tokens, int32_t num_heads,
+                            int32_t num_kv_heads, int32_t head_dim, int64_t num_slots);
+
 #ifdef __cplusplus
 }  /* extern "C" */
 #endif

@@ -37,6 +37,10 @@ SYMBOLS = {
         _c.c_void_p, _c.c_void_p, _c.c_size_t,
         _c.c_int32, _c.c_int32, _c.c_int32, _c.c_int32, _c.c_int32, _c.c_int32,
         _c.c_int32, _c.c_float, _c.c_int32, _c.c_uint32]),
+    "nvj_qk_norm_rope_store_launch": (_c.c_int, [
+        _c.c_void_p, _c.c_void_p, _c.c_int64, _c.c_void_p, _c.c_void_p, _c.c_int32, _c.c_void_p,
+        _c.c_void_p, _c.c_float, _c.c_void_p, _c.c_void_p, _c.c_void_p, _c.c_void_p,
+        _c.c_int32, _c.c_int32, _c.c_int32, _c.c_int32, _c.c_int64]),
 }
 NVJ_PHASE_SPLITK = 1
 NVJ_PHASE_COMBINE = 2

@@ -25,7 +25,8 @@ import torch
 import torch.nn.functional as F
 
 from ..layers.attention import Attention
-from ..layers.paged_attention import paged_decode_workspace_bytes
+from ..layers.paged_attention import paged_attention, paged_decode_workspace_bytes
+from ..layers.qk_rope_store import qk_norm_rope_store
 from ..utils.context import AttentionContext, create_decode_context
 
 __all__ = ["DecodeModelConfig", "DecodeStepRunner", "prepare_block_tables", "prepare_decode"]
@@ -79,8 +80,11 @@ class DecodeStepRunner:
     ``Attention`` per layer; ``step`` runs one decode step for a batch."""
 
     def __init__(self, cfg: DecodeModelConfig, device="cuda:0", seed: int = 0,
-                 fill_cache: bool = True):
+                 fill_cache: bool = True, fused_qk_rope_store: bool = True):
         self.cfg = cfg
+        # True: one HIP launch for QK-RMSNorm + RoPE + KV store; False: the
+        # reference's op-by-op chain in torch followed by the plain store
+        self.fused_qk_rope_store = fused_qk_rope_store
         self.device = torch.device(device)
         g = torch.Generator(device=self.device)
         g.manual_seed(seed)
@@ -157,6 +161,19 @@ class DecodeStepRunner:
             else:
                 h, residual = self._rms(h, lw["ln1"], residual)
             qkv = F.linear(h, lw["qkv"])
+            if self.fused_qk_rope_store:
+                q = qk_norm_rope_store(qkv, positions, self.cos_sin, lw["q_norm"], lw["k_norm"],
+                                       c.rms_norm_eps, attn.k_cache, attn.v_cache,
+                                       context.slot_mapping, c.num_heads, c.num_kv_heads,
+                                       c.head_dim)
+                o = paged_attention(q, attn.k_cache, attn.v_cache, context.block_tables,
+                                    context.context_lens, attn.scale, attn.block_size,
+                                    workspace=attn.workspace)
+                h = F.linear(o.reshape(-1, qs), lw["o"])
+                h, residual = self._rms(h, lw["ln2"], residual)
+                gate, up = F.linear(h, lw["gate_up"]).chunk(2, dim=-1)
+                h = F.linear(F.silu(gate) * up, lw["down"])
+                continue
             q, k, v = qkv.split([qs, ks, ks], dim=-1)
             q = q.reshape(-1, c.num_heads, c.head_dim)
             k = k.reshape(-1, c.num_kv_heads, c.head_dim)

@@ -21,6 +21,15 @@ What pins each function (see tests/test_oracle_pinning.py):
                                   closed forms (ctx=1 -> V row, equal keys ->
                                   mean of V, ctx=0 -> zeros), permutation and
                                   padding invariance.
+* ``qk_norm_rope_ref`` / ``qk_norm_rope_store_ref`` / ``build_cos_sin_cache_ref``
+                                - float64 RMSNorm and rotation; closed forms
+                                  (position 0 is the identity, unit weight gives
+                                  unit RMS, rotation preserves each pair's norm,
+                                  q.k depends on the position difference only).
+                                  The fp32 summation order of the mean is this
+                                  oracle's choice (the reference leaves it to
+                                  XLA): PARITY UNPINNED at the level of fp32
+                                  round-off of that sum.
 * ``paged_attention_fallback_ref``
                                 - same checks; the bf16 rounding of the
                                   probabilities inside ``jax.nn.dot_product_attention``
@@ -44,6 +53,9 @@ __all__ = [
     "paged_decode_attention_per_seq_ref",
     "paged_attention_fallback_ref",
     "textbook_attention_f64",
+    "build_cos_sin_cache_ref",
+    "qk_norm_rope_ref",
+    "qk_norm_rope_store_ref",
 ]
 
 
@@ -294,3 +306,84 @@ def textbook_attention_f64(q, k_cache, v_cache, block_tables, context_lens,
                 acc += w[pos] * vf[page, pos % block_size, kvh]
             out[b, h] = acc
     return out
+
+
+# ---------------------------------------------------------------------------
+# QK-RMSNorm + rotary embedding (+ store): the ops in front of the path
+# ---------------------------------------------------------------------------
+
+def build_cos_sin_cache_ref(head_dim: int, max_position: int, base: float) -> np.ndarray:
+    """``RotaryEmbedding.__init__`` (``layers/rotary_embedding.py:60-76``):
+    ``inv_freq = 1 / base ** (arange(0, D, 2) / D)``, ``freqs = outer(t, inv_freq)``,
+    cache = ``[cos(freqs) | sin(freqs)]`` as float32 ``[max_position, D]``."""
+    inv_freq = (1.0 / (np.float32(base) ** (np.arange(0, head_dim, 2, dtype=np.float32)
+                                            / np.float32(head_dim)))).astype(np.float32)
+    t = np.arange(max_position, dtype=np.float32)
+    freqs = np.einsum("i,j->ij", t, inv_freq).astype(np.float32)
+    return np.concatenate([np.cos(freqs), np.sin(freqs)], axis=-1).astype(np.float32)
+
+
+def _butterfly_sum_128(sq1: np.ndarray, sq2: np.ndarray) -> np.ndarray:
+    """Sum of 128 squares in the order the HIP kernel uses: lane l starts from
+    x[l]^2 + x[l+64]^2, then adds its xor partner for masks 32, 16, .., 1.
+    fp32 throughout; every lane ends with the same value, lane 0 is returned."""
+    s = (sq1 + sq2).astype(np.float32)                  # [..., 64]
+    lanes = np.arange(64)
+    for m in (32, 16, 8, 4, 2, 1):
+        s = (s + s[..., lanes ^ m]).astype(np.float32)
+    return s[..., :1]
+
+
+def qk_norm_rope_ref(x, positions, cos_sin_cache, weight, eps):
+    """RMSNorm over the head dimension, then rotary embedding, for q or k.
+
+    x : [T, H, 128] bf16 bits.  Follows ``RMSNorm._rms_forward``
+    (``layers/layernorm.py:31-48``: fp32, ``x * rsqrt(mean(x^2) + eps) * weight``,
+    cast back to the input dtype) and ``apply_rotary_emb``
+    (``layers/rotary_embedding.py:13-37``: halves ``x1, x2``; ``y1 = x1 cos - x2
+    sin``, ``y2 = x2 cos + x1 sin`` with float32 cos/sin, so the result is
+    float32), with ``cos_sin = cache[positions]`` (:96-106).  ``weight`` None
+    skips the norm (``models/qwen3.py:157``).  Returns float32 ``[T, H, 128]``.
+
+    The reference leaves the fp32 summation order of the mean to XLA; this
+    restatement fixes it to the xor-butterfly order of the HIP kernel so that
+    the two agree bit for bit.  Any other order differs by fp32 round-off only.
+    """
+    xf = bf16_bits_to_f32(np.asarray(x))
+    T, H, D = xf.shape
+    assert D == 128
+    x1, x2 = xf[..., :64], xf[..., 64:]
+    if weight is not None:
+        w = np.asarray(weight, dtype=np.float32)
+        s = _butterfly_sum_128(x1 * x1, x2 * x2)
+        var = s * np.float32(1.0 / 128.0) + np.float32(eps)
+        r = (np.float32(1.0) / np.sqrt(var, dtype=np.float32)).astype(np.float32)
+        x1 = bf16_bits_to_f32(f32_to_bf16_bits((x1 * r) * w[:64]))
+        x2 = bf16_bits_to_f32(f32_to_bf16_bits((x2 * r) * w[64:]))
+    pos = np.clip(np.asarray(positions, dtype=np.int64), 0, cos_sin_cache.shape[0] - 1)
+    cs = np.asarray(cos_sin_cache, dtype=np.float32)[pos][:, None, :]
+    cos, sin = cs[..., :64], cs[..., 64:]
+    y1 = (x1 * cos).astype(np.float32) - (x2 * sin).astype(np.float32)
+    y2 = (x2 * cos).astype(np.float32) + (x1 * sin).astype(np.float32)
+    return np.concatenate([y1, y2], axis=-1).astype(np.float32)
+
+
+def qk_norm_rope_store_ref(qkv, positions, cos_sin_cache, q_weight, k_weight, eps, k_cache,
+                           v_cache, slot_mapping, num_heads, num_kv_heads,
+                           negative_slots: str = "skip"):
+    """The chain ``models/qwen3.py:150-166`` + ``layers/attention.py:386-387, 457-475``
+    for packed ``qkv`` [T, (Hq + 2 Hkv) * 128] bf16 bits: split, QK norm, RoPE,
+    q cast to bf16, K (float32 after RoPE) and V stored through
+    ``store_kv_to_cache_ref``.  Returns ``(q_bits, k_cache, v_cache)``."""
+    qkv = np.asarray(qkv)
+    T = qkv.shape[0]
+    D = 128
+    qs, ks = num_heads * D, num_kv_heads * D
+    q = qkv[:, :qs].reshape(T, num_heads, D)
+    k = qkv[:, qs:qs + ks].reshape(T, num_kv_heads, D)
+    v = qkv[:, qs + ks:qs + 2 * ks].reshape(T, num_kv_heads, D)
+    q_rot = qk_norm_rope_ref(q, positions, cos_sin_cache, q_weight, eps)
+    k_rot = qk_norm_rope_ref(k, positions, cos_sin_cache, k_weight, eps)
+    kc, vc = store_kv_to_cache_ref(k_rot, np.ascontiguousarray(v), k_cache, v_cache,
+                                   slot_mapping, negative_slots=negative_slots)
+    return f32_to_bf16_bits(q_rot), kc, vc

@@ -11,12 +11,12 @@ from helpers import bits_to_torch, torch_to_bits
 pytestmark = pytest.mark.gpu
 
 
-def _small_runner():
+def _small_runner(fused=True):
     from nanovllm_jax_amd.engine.decode_step import DecodeModelConfig, DecodeStepRunner
     cfg = DecodeModelConfig(num_layers=2, hidden_size=256, num_heads=4, num_kv_heads=2,
                             head_dim=128, intermediate_size=512, vocab_size=1024,
                             max_position=2048, block_size=256, num_kvcache_blocks=12)
-    return cfg, DecodeStepRunner(cfg, "cuda:0", seed=3)
+    return cfg, DecodeStepRunner(cfg, "cuda:0", seed=3, fused_qk_rope_store=fused)
 
 
 def _batch(cfg):
@@ -81,10 +81,11 @@ def _cpu_reference(runner, cfg, ids, pos, ctx_lens, slots, bt):
     return h @ f(runner.embed).T
 
 
-def test_decode_step_matches_cpu_model_with_oracle_attention():
-    print("case decode step vs CPU model", flush=True)
+@pytest.mark.parametrize("fused", [True, False])
+def test_decode_step_matches_cpu_model_with_oracle_attention(fused):
+    print(f"case decode step vs CPU model fused={fused}", flush=True)
     from nanovllm_jax_amd.engine.decode_step import prepare_decode
-    cfg, runner = _small_runner()
+    cfg, runner = _small_runner(fused)
     last, lens, tables = _batch(cfg)
     ids, pos, ctx_lens, slots, bt = prepare_decode(last, lens, tables, cfg.block_size)
     want = _cpu_reference(runner, cfg, ids, pos, ctx_lens, slots, bt)   # before the step mutates the cache

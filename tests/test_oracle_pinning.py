@@ -201,3 +201,91 @@ def test_restatements_agree_with_each_other_at_c1():
     np.testing.assert_allclose(v, a, atol=1e-6, rtol=2 ** -8)
     f = bf16_bits_to_f32(paged_attention_fallback_ref(*args))
     np.testing.assert_allclose(f, a, atol=1e-2, rtol=1e-2)     # the path's parity bar
+
+
+# ---------------------------------------------------------------- QK norm + RoPE
+def _rope_inputs(seed, T=6, H=3):
+    from oracle.paged_attention_oracle import build_cos_sin_cache_ref
+    rng = np.random.Generator(np.random.PCG64(seed))
+    x = f32_to_bf16_bits(rng.standard_normal((T, H, 128), dtype=np.float32) * 3)
+    w = (1 + 0.1 * rng.standard_normal(128)).astype(np.float32)
+    pos = rng.integers(0, 4096, T).astype(np.int32)
+    return x, w, pos, build_cos_sin_cache_ref(128, 4096, 1e6)
+
+
+def test_cos_sin_cache_against_float64():
+    from oracle.paged_attention_oracle import build_cos_sin_cache_ref
+    cs = build_cos_sin_cache_ref(128, 512, 1e6)
+    inv = 1.0 / (1e6 ** (np.arange(0, 128, 2, dtype=np.float64) / 128))
+    f = np.outer(np.arange(512, dtype=np.float64), inv)
+    assert cs.shape == (512, 128) and cs.dtype == np.float32
+    np.testing.assert_allclose(cs[:, :64], np.cos(f), atol=3e-5)
+    np.testing.assert_allclose(cs[:, 64:], np.sin(f), atol=3e-5)
+    assert np.array_equal(cs[0, :64], np.ones(64, np.float32)) and not cs[0, 64:].any()
+
+
+def test_qk_norm_rope_against_float64_math():
+    from oracle.paged_attention_oracle import qk_norm_rope_ref
+    x, w, pos, cs = _rope_inputs(61)
+    got = qk_norm_rope_ref(x, pos, cs, w, 1e-6)
+    xf = bf16_bits_to_f32(x).astype(np.float64)
+    n = xf / np.sqrt((xf ** 2).mean(-1, keepdims=True) + 1e-6) * w
+    c = cs[pos][:, None, :64].astype(np.float64); s = cs[pos][:, None, 64:].astype(np.float64)
+    want = np.concatenate([n[..., :64] * c - n[..., 64:] * s, n[..., 64:] * c + n[..., :64] * s], -1)
+    # the normalised value is rounded to bf16 before the rotation: 2^-8 relative
+    np.testing.assert_allclose(got, want, atol=2e-2, rtol=2 ** -7)
+    # without the norm only fp32 round-off remains
+    got2 = qk_norm_rope_ref(x, pos, cs, None, 1e-6)
+    want2 = np.concatenate([xf[..., :64] * c - xf[..., 64:] * s, xf[..., 64:] * c + xf[..., :64] * s], -1)
+    np.testing.assert_allclose(got2, want2, atol=1e-5, rtol=1e-6)
+
+
+def test_qk_norm_rope_closed_forms():
+    from oracle.paged_attention_oracle import qk_norm_rope_ref
+    x, w, pos, cs = _rope_inputs(62)
+    ones = np.ones(128, np.float32)
+    zero = np.zeros_like(pos)
+    # position 0: cos = 1, sin = 0 -> rotation is the identity
+    assert np.array_equal(qk_norm_rope_ref(x, zero, cs, None, 1e-6), bf16_bits_to_f32(x))
+    # unit weight -> unit RMS (up to the bf16 rounding of the normalised value)
+    y = qk_norm_rope_ref(x, pos, cs, ones, 1e-6)
+    np.testing.assert_allclose(np.sqrt((y.astype(np.float64) ** 2).mean(-1)), 1.0, atol=3e-3)
+    # the rotation preserves the norm of every (i, i + 64) pair
+    y0 = qk_norm_rope_ref(x, pos, cs, None, 1e-6).astype(np.float64)
+    xf = bf16_bits_to_f32(x).astype(np.float64)
+    np.testing.assert_allclose(y0[..., :64] ** 2 + y0[..., 64:] ** 2,
+                               xf[..., :64] ** 2 + xf[..., 64:] ** 2, rtol=1e-5, atol=1e-6)
+    # q . k after rotation depends on the position difference only
+    q = x[:1, :1]; k = x[1:2, :1]
+    def dot(pq, pk):
+        a = qk_norm_rope_ref(q, np.array([pq]), cs, None, 0).astype(np.float64)
+        b = qk_norm_rope_ref(k, np.array([pk]), cs, None, 0).astype(np.float64)
+        return float((a * b).sum())
+    assert abs(dot(100, 40) - dot(1060, 1000)) < 1e-2 * (1 + abs(dot(100, 40)))
+    assert abs(dot(100, 40) - dot(100, 41)) > 1e-3
+    # out-of-range positions are clamped like a JAX gather
+    big = np.array([10 ** 6] * len(pos))
+    assert np.array_equal(qk_norm_rope_ref(x, big, cs, w, 1e-6),
+                          qk_norm_rope_ref(x, np.full(len(pos), 4095), cs, w, 1e-6))
+
+
+def test_qk_norm_rope_store_composes_the_pieces():
+    from oracle.paged_attention_oracle import qk_norm_rope_ref, qk_norm_rope_store_ref
+    rng = np.random.Generator(np.random.PCG64(63))
+    T, Hq, Hkv = 5, 4, 2
+    _, w, pos, cs = _rope_inputs(64, T=T)
+    qkv = f32_to_bf16_bits(rng.standard_normal((T, (Hq + 2 * Hkv) * 128), dtype=np.float32))
+    kc = rng.integers(0, 65536, (16, Hkv, 128)).astype(np.uint16)
+    vc = rng.integers(0, 65536, (16, Hkv, 128)).astype(np.uint16)
+    slots = np.array([3, -1, 15, 16, 0], np.int32)
+    q, k2, v2 = qk_norm_rope_store_ref(qkv, pos, cs, w, w[::-1].copy(), 1e-6, kc, vc, slots, Hq, Hkv)
+    qh = qkv[:, :Hq * 128].reshape(T, Hq, 128)
+    kh = qkv[:, Hq * 128:(Hq + Hkv) * 128].reshape(T, Hkv, 128)
+    vh = qkv[:, (Hq + Hkv) * 128:].reshape(T, Hkv, 128)
+    assert np.array_equal(q, f32_to_bf16_bits(qk_norm_rope_ref(qh, pos, cs, w, 1e-6)))
+    kr = f32_to_bf16_bits(qk_norm_rope_ref(kh, pos, cs, w[::-1].copy(), 1e-6))
+    for t, s in enumerate(slots):
+        if 0 <= s < 16:
+            assert np.array_equal(k2[s], kr[t]) and np.array_equal(v2[s], vh[t])
+    untouched = [i for i in range(16) if i not in (3, 15, 0)]
+    assert np.array_equal(k2[untouched], kc[untouched]) and np.array_equal(v2[untouched], vc[untouched])
