@@ -99,15 +99,15 @@ class DecodeStepRunner:
         self.layers = []
         for _ in range(c.num_layers):
             self.layers.append(dict(
-                ln1=torch.ones(c.hidden_size, device=self.device),
-                ln2=torch.ones(c.hidden_size, device=self.device),
+                ln1=torch.ones(c.hidden_size, device=self.device, dtype=torch.bfloat16),
+                ln2=torch.ones(c.hidden_size, device=self.device, dtype=torch.bfloat16),
                 qkv=w(qkv_out, c.hidden_size),
                 o=w(c.hidden_size, c.num_heads * c.head_dim),
                 q_norm=torch.ones(c.head_dim, device=self.device),
                 k_norm=torch.ones(c.head_dim, device=self.device),
                 gate_up=w(2 * c.intermediate_size, c.hidden_size),
                 down=w(c.hidden_size, c.intermediate_size)))
-        self.final_norm = torch.ones(c.hidden_size, device=self.device)
+        self.final_norm = torch.ones(c.hidden_size, device=self.device, dtype=torch.bfloat16)
         inv_freq = 1.0 / (c.rope_theta ** (torch.arange(0, c.head_dim, 2, dtype=torch.float32,
                                                         device=self.device) / c.head_dim))
         freqs = torch.outer(torch.arange(c.max_position, dtype=torch.float32,
@@ -132,15 +132,13 @@ class DecodeStepRunner:
 
     # -- small torch pieces -------------------------------------------------
     def _rms(self, x, weight, residual=None):
-        """RMSNorm, optionally fused with the residual add (layernorm.py:31-79)."""
+        """RMSNorm, optionally fused with the residual add (layernorm.py:31-79):
+        the sum is taken in fp32 and rounded once to the model dtype, which is
+        both the new residual and the input of the norm (the reference norms
+        the unrounded fp32 sum; the difference is one bf16 rounding)."""
         if residual is not None:
-            xf = x.float() + residual.float()
-            residual = xf.to(x.dtype)
-        else:
-            xf = x.float()
-            residual = x
-        var = xf.pow(2).mean(-1, keepdim=True)
-        return (xf * torch.rsqrt(var + self.cfg.rms_norm_eps) * weight).to(x.dtype), residual
+            x = (x.float() + residual.float()).to(x.dtype)
+        return F.rms_norm(x, (x.shape[-1],), weight.to(x.dtype), self.cfg.rms_norm_eps), x
 
     def _rope(self, x, cos, sin):
         """x bf16 [T, H, D]; result float32 like the reference's promotion
