@@ -32,7 +32,7 @@ HBM_PEAK_GBPS = 8000.0
 # this very command, scaled by the same counters over a plain 1 GiB copy
 # (FETCH_SIZE x1.9999, WRITE_SIZE x1.0).  Keyed by (workload, chunk); other
 # configurations report null.
-MEASURED_TRAFFIC_BYTES = {("C2", 1024): 1_080_188_000}
+MEASURED_TRAFFIC_BYTES = {("C2", 0): 1_080_188_000, ("C2", 1024): 1_080_188_000}
 
 
 def device_inputs(w, torch, dev):
@@ -164,7 +164,8 @@ def main():
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--workload", default="C2", choices=["C1", "C2", "C3", "C4", "C5"])
-    ap.add_argument("--chunk", type=int, default=0, help="positions per workgroup (0 = default)")
+    ap.add_argument("--chunk", type=int, default=0,
+                    help="positions per workgroup (0 = balanced split, the default)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run a plain 1 GiB device-to-device copy a few times, so a "
@@ -186,8 +187,7 @@ def main():
               file=sys.stderr)
         return 1
     from nanovllm_jax_amd import _lib, paged_attention, store_kv_to_cache
-    from nanovllm_jax_amd.layers.paged_attention import (default_chunk,
-                                                         paged_decode_workspace_bytes)
+    from nanovllm_jax_amd.layers.paged_attention import paged_decode_workspace_bytes
     from nanovllm_jax_amd.workloads import algorithmic_bytes, make_workload
 
     dev = torch.device("cuda:0")
@@ -196,7 +196,7 @@ def main():
         return bench_decode_step(args, torch)
     w = make_workload(args.workload)
     q, kc, vc, bt, ctx, slots, k_new, v_new = device_inputs(w, torch, dev)
-    chunk = args.chunk or default_chunk(w.batch, w.num_kv_heads, w.max_blocks, w.block_size)
+    chunk = args.chunk
     ws = torch.empty(paged_decode_workspace_bytes(w.batch, w.num_heads, w.head_dim, w.max_blocks,
                                                   w.block_size, w.num_kv_heads, chunk),
                      dtype=torch.uint8, device=dev)
@@ -243,7 +243,8 @@ def main():
                                f"D={w.head_dim} page={w.block_size} "
                                f"ctx={int(w.context_lens.min())}..{int(w.context_lens.max())} "
                                f"pool={w.num_blocks} pages",
-                   "chunk": chunk, "algorithmic_bytes_per_call": byts,
+                   "split": "balanced" if chunk == 0 else f"fixed chunk {chunk}",
+                   "algorithmic_bytes_per_call": byts,
                    "step": "split-K launch + combine launch"},
         "roofline": {"bound": "hbm", "achieved": round(gbps_kernel, 1), "peak": HBM_PEAK_GBPS,
                      "unit": "GB/s", "frac": round(gbps_kernel / HBM_PEAK_GBPS, 4),

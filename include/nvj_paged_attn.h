@@ -72,17 +72,29 @@ NVJ_API int nvj_store_kvcache_launch(void* stream,
                              int32_t k_dtype, int32_t v_dtype);
 
 /*
- * Split size (positions of one sequence handled by one workgroup) the library
- * would pick for this problem when the caller passes chunk == 0.  Always a
- * multiple of 32.
+ * How the positions of a call are split over workgroups is chosen by `chunk`:
+ *
+ *   chunk == 0  balanced split (the default): the 32-position steps of all
+ *               sequences, end to end in batch order, are cut into equal runs,
+ *               one per workgroup and at most one workgroup per CU (256), at
+ *               least 128 positions each.  The kernel derives the cut from
+ *               context_lens on the device, so ragged batches are balanced
+ *               without the host knowing the lengths.
+ *   chunk  > 0  fixed split: workgroup (b, c) takes positions
+ *               [c * chunk, (c + 1) * chunk) of sequence b; chunk must be a
+ *               multiple of 32.
+ *
+ * nvj_paged_decode_default_chunk: the fixed chunk the library recommends for a
+ * problem of this shape when a fixed split is wanted (a multiple of 32).
  */
 NVJ_API int32_t nvj_paged_decode_default_chunk(int32_t batch, int32_t num_kv_heads,
                                        int32_t max_blocks, int32_t block_size);
 
 /*
- * Bytes of device workspace nvj_paged_decode_launch needs for the split-K
- * partials (fp32 accumulators plus running max and sum per split).  chunk == 0
- * means the default chunk.  Returns 0 on invalid arguments.
+ * Bytes of device workspace nvj_paged_decode_launch needs for the partials
+ * (fp32 accumulators plus running max and sum per partial; in balanced mode
+ * also batch + 1 int32 prefix sums) for the given `chunk` mode.  Returns 0 on
+ * invalid arguments.
  */
 NVJ_API size_t nvj_paged_decode_workspace_bytes(int32_t batch, int32_t num_heads,
                                         int32_t head_dim, int32_t max_blocks,
@@ -114,10 +126,10 @@ NVJ_API size_t nvj_paged_decode_workspace_bytes(int32_t batch, int32_t num_heads
  * [0, num_blocks); the kernel clamps them into range like the reference (:185)
  * rather than faulting.
  *
- * Two launches on `stream`: the split-K kernel (one workgroup per
- * (sequence, chunk of positions), all KV heads) and the combine pass.
+ * Two launches on `stream`: the split-K kernel (each workgroup streams its
+ * share of positions for all KV heads) and the combine pass.
  * Supported: head_dim 128, num_heads / num_kv_heads <= 16, block_size a
- * multiple of 32, chunk a multiple of 32 (0 = default).
+ * multiple of 32, chunk a multiple of 32 (0 = balanced split).
  */
 NVJ_API int nvj_paged_decode_launch(void* stream,
                             const void* q, const void* k_cache, const void* v_cache,

@@ -56,19 +56,10 @@ __device__ __forceinline__ float wave_xor_max(float x, int mask) {
   return fmaxf(x, __shfl_xor(x, mask, 64));
 }
 
-// Byte offset of load slot `x` (position within the step) for this lane, as a
-// 32-bit quantity: a step never leaves its page, so it is below
-// block_size * row_bytes.  TAIL steps clamp the slot to the last live position
-// so nothing at or beyond the context length is ever read.
-template <bool TAIL>
-__device__ __forceinline__ uint32_t slot_offset(int x, int last, uint32_t row_bytes,
-                                                uint32_t lane_bytes) {
-  if constexpr (TAIL) x = min(x, last);
-  return (uint32_t)x * row_bytes + lane_bytes;
-}
-
 // K/V are read exactly once per call: non-temporal loads stream them past the
-// caches instead of allocating lines that will never be hit again.
+// caches instead of allocating lines that will never be hit again.  `base` is
+// wave-uniform (scalar registers), `off` the lane's 32-bit byte offset: a step
+// never leaves its page, so offsets stay below block_size * row_bytes.
 __device__ __forceinline__ uint4 load_piece(const char* base, uint32_t off) {
   typedef __attribute__((ext_vector_type(4))) unsigned int u32x4;
   const u32x4 t = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(base + off));
@@ -76,14 +67,24 @@ __device__ __forceinline__ uint4 load_piece(const char* base, uint32_t off) {
 }
 
 // K of one step: load slot i of lane (kg, r) is position 4*i + kg, piece r, so
-// a quarter-wave reads one whole 256-byte (position, head) row.
+// a quarter-wave reads one whole 256-byte (position, head) row.  In a full
+// step the position splits into a uniform part (4*i rows, folded into the
+// scalar base) and one per-lane offset shared by all 8 loads; a TAIL step
+// clamps every slot to the last live position so that nothing at or beyond
+// the context length is ever read.
 template <bool TAIL>
 __device__ __forceinline__ void issue_k_loads(uint4 (&kreg)[8], const char* base, int kg,
                                               int last, uint32_t row_bytes,
                                               uint32_t lane_bytes) {
 #pragma unroll
-  for (int i = 0; i < 8; ++i)
-    kreg[i] = load_piece(base, slot_offset<TAIL>(4 * i + kg, last, row_bytes, lane_bytes));
+  for (int i = 0; i < 8; ++i) {
+    if constexpr (TAIL) {
+      kreg[i] = load_piece(base, (uint32_t)min(4 * i + kg, last) * row_bytes + lane_bytes);
+    } else {
+      kreg[i] = load_piece(base + (size_t)(4 * i) * row_bytes,
+                           (uint32_t)kg * row_bytes + lane_bytes);
+    }
+  }
 }
 
 // V of one step: load slot j of lane (kg, r) is the position that reduction
@@ -95,39 +96,53 @@ __device__ __forceinline__ void issue_v_loads(uint4 (&vreg)[8], const char* base
                                               uint32_t lane_bytes) {
 #pragma unroll
   for (int j = 0; j < 8; ++j) {
-    const int x = (j < 4) ? (4 * kg + j) : (16 + 4 * kg + (j - 4));
-    vreg[j] = load_piece(base, slot_offset<TAIL>(x, last, row_bytes, lane_bytes));
+    const int uni = (j < 4) ? j : (16 + j - 4);   // uniform part of the position
+    if constexpr (TAIL) {
+      vreg[j] = load_piece(base, (uint32_t)min(4 * kg + uni, last) * row_bytes + lane_bytes);
+    } else {
+      vreg[j] = load_piece(base + (size_t)uni * row_bytes,
+                           (uint32_t)(4 * kg) * row_bytes + lane_bytes);
+    }
   }
 }
 
-// grid.x = batch * max_chunks, grid.y = num_kv_heads / NW, block = NW * 64.
-template <int NW>
-__global__ __launch_bounds__(NW * 64) void paged_decode_splitk_kernel(
-    const uint4* __restrict__ q,          // [B, Hq, 16] pieces
-    const char* __restrict__ k_cache,     // [NB, bs, Hkv, 128] bf16
-    const char* __restrict__ v_cache,
-    const int32_t* __restrict__ block_tables,  // [B, MB]
-    const int32_t* __restrict__ context_lens,  // [B]
-    uint4* __restrict__ out,              // [B, Hq, 16] pieces (bf16)
-    float* __restrict__ part_o,           // [B, max_chunks, Hq, 128]
-    float* __restrict__ part_ml,          // [B, max_chunks, Hq, 2]
-    int num_heads, int num_kv_heads, int group, int block_size, int max_blocks,
-    int num_blocks, int chunk, int max_chunks, float scale_log2e) {
-  __shared__ uint4 k_tile[NW][kStep * kLdsRowPieces];
+// Read-only int32 metadata (block tables, context lengths) is never written
+// while a launch runs.  Reading it through the constant address space tells
+// the compiler so: a wave-uniform index then becomes a scalar load (s_load)
+// even after the kernel has issued stores of its own, instead of a vector load
+// whose result has to be moved back to the scalar unit.
+typedef const __attribute__((address_space(4))) int32_t* const_i32_ptr;
+__device__ __forceinline__ const_i32_ptr as_constant(const int32_t* p) {
+  return (const_i32_ptr)(uintptr_t)p;
+}
 
-  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-  const int lane = threadIdx.x & 63;
-  const int r = lane & 15;   // MFMA row/column index inside a 16-wide tile
-  const int kg = lane >> 4;  // MFMA k-group (which 8 of the 32 reduction slots)
+// Everything shared by the launch: pointers and problem shape.
+struct DecodeArgs {
+  const uint4* q;              // [B, Hq, 16] pieces
+  const char* k_cache;         // [NB, bs, Hkv, 128] bf16
+  const char* v_cache;
+  const int32_t* block_tables; // [B, MB]
+  const int32_t* context_lens; // [B]
+  uint4* out;                  // [B, Hq, 16] pieces (bf16)
+  float* part_o;               // [slots, Hq, 128]
+  float* part_ml;              // [slots, Hq, 2]
+  int num_heads, num_kv_heads, group, block_size, max_blocks, num_blocks;
+  float scale_log2e;
+};
 
-  const int b = blockIdx.x / max_chunks;
-  const int c = blockIdx.x - b * max_chunks;
-  // A length beyond what the block table can describe is clamped to it.
-  const int ctx = min(context_lens[b], max_blocks * block_size);
-  const int t0 = c * chunk;
-  if (t0 >= ctx) return;  // also every chunk of an empty sequence
-  const int t1 = min(ctx, t0 + chunk);
-  const int kvh = blockIdx.y * NW + wave;
+// One wave's share of one segment: positions [t0, t1) of sequence b for KV head
+// kvh.  `direct` means the segment is the whole sequence: the normalised bf16
+// result goes straight to `out`; otherwise the unnormalised partial goes to
+// partial slot `slot` of the workspace.  t0 is a multiple of 32, t0 < t1.
+__device__ __forceinline__ void run_segment(const DecodeArgs& a, uint4* lds, int b, int kvh,
+                                            int t0, int t1, int64_t slot, bool direct, int r,
+                                            int kg) {
+  const uint4* __restrict__ q = a.q;
+  const char* __restrict__ k_cache = a.k_cache;
+  const char* __restrict__ v_cache = a.v_cache;
+  const int num_heads = a.num_heads, group = a.group, block_size = a.block_size;
+  const int num_blocks = a.num_blocks;
+  const float scale_log2e = a.scale_log2e;
   const int nsteps = (t1 - t0 + kStep - 1) / kStep;
 
   // Q^T as MFMA B operand for the 4 reduction steps over head_dim:
@@ -135,17 +150,22 @@ __global__ __launch_bounds__(NW * 64) void paged_decode_splitk_kernel(
   // 32*s + 8*kg .. +8.  Columns >= group are zero.
   bf16x8 qreg[4];
   {
+    // lanes of padding columns read the group's last head (always in range)
+    // and then drop it, so the loads stay unconditional 16-byte loads
     const uint4 zero = make_uint4(0u, 0u, 0u, 0u);
-    const uint4* qrow = q + ((int64_t)b * num_heads + (int64_t)kvh * group + r) * kRowPieces;
+    const uint4* qrow =
+        q + ((int64_t)b * num_heads + (int64_t)kvh * group + min(r, group - 1)) * kRowPieces;
 #pragma unroll
-    for (int s = 0; s < 4; ++s) qreg[s] = as_bf16x8(r < group ? qrow[4 * s + kg] : zero);
+    for (int s = 0; s < 4; ++s) {
+      const uint4 v = qrow[4 * s + kg];
+      qreg[s] = as_bf16x8(r < group ? v : zero);
+    }
   }
 
-  const uint32_t row_bytes = (uint32_t)num_kv_heads * (kHeadDim * 2);  // one position, all heads
+  const uint32_t row_bytes = (uint32_t)a.num_kv_heads * (kHeadDim * 2);  // one position, all heads
   const uint32_t lane_bytes = (uint32_t)r * 16u;
   const int64_t head_bytes = (int64_t)kvh * (kHeadDim * 2);
-  const int32_t* table = block_tables + (int64_t)b * max_blocks;
-  uint4* lds = k_tile[wave];
+  const const_i32_ptr table = as_constant(a.block_tables + (int64_t)b * a.max_blocks);
 
   // wave-uniform byte offset of the first position of a step inside the cache
   auto step_base = [&](int step) -> int64_t {
@@ -271,10 +291,9 @@ __global__ __launch_bounds__(NW * 64) void paged_decode_splitk_kernel(
   if (r >= group) return;
   const int head = kvh * group + r;
   // acc[jd][e] is O[head][dim = 32*kg + 8*e + jd]
-  const int nchunks = (ctx + chunk - 1) / chunk;
-  if (nchunks == 1) {
+  if (direct) {
     const float inv = 1.0f / (l_run + 1e-9f);
-    uint4* orow = out + ((int64_t)b * num_heads + head) * kRowPieces + 4 * kg;
+    uint4* orow = a.out + ((int64_t)b * num_heads + head) * kRowPieces + 4 * kg;
 #pragma unroll
     for (int e = 0; e < 4; ++e) {
       uint4 o;
@@ -285,45 +304,230 @@ __global__ __launch_bounds__(NW * 64) void paged_decode_splitk_kernel(
       orow[e] = o;
     }
   } else {
-    const int64_t slot = ((int64_t)b * max_chunks + c) * num_heads + head;
-    float4* prow = reinterpret_cast<float4*>(part_o + slot * kHeadDim + 32 * kg);
+    const int64_t row = slot * num_heads + head;
+    float4* prow = reinterpret_cast<float4*>(a.part_o + row * kHeadDim + 32 * kg);
 #pragma unroll
     for (int e = 0; e < 4; ++e) {
       prow[2 * e] = make_float4(acc[0][e], acc[1][e], acc[2][e], acc[3][e]);
       prow[2 * e + 1] = make_float4(acc[4][e], acc[5][e], acc[6][e], acc[7][e]);
     }
-    if (kg == 0) {
-      reinterpret_cast<float2*>(part_ml)[slot] = make_float2(m_run, l_run);
-    }
+    if (kg == 0) reinterpret_cast<float2*>(a.part_ml)[row] = make_float2(m_run, l_run);
   }
 }
 
-// Merge the per-chunk partials of one (sequence, query head).  grid = (B, Hq),
-// block = 128 lanes, one per output dim.
+// Fixed-chunk split: grid.x = batch * max_chunks, grid.y = num_kv_heads / NW,
+// block = NW * 64.  Workgroup (b, c) owns positions [c*chunk, (c+1)*chunk) of
+// sequence b; partial slot = b * max_chunks + c.
+template <int NW>
+__global__ __launch_bounds__(NW * 64) void paged_decode_splitk_kernel(DecodeArgs a, int chunk,
+                                                                      int max_chunks) {
+  __shared__ uint4 k_tile[NW][kStep * kLdsRowPieces];
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int lane = threadIdx.x & 63;
+  const int b = blockIdx.x / max_chunks;
+  const int c = blockIdx.x - b * max_chunks;
+  // A length beyond what the block table can describe is clamped to it.
+  const int ctx = min(a.context_lens[b], a.max_blocks * a.block_size);
+  const int t0 = c * chunk;
+  if (t0 >= ctx) return;  // also every chunk of an empty sequence
+  const int t1 = min(ctx, t0 + chunk);
+  const bool direct = ctx <= chunk;
+  run_segment(a, k_tile[wave], b, blockIdx.y * NW + wave, t0, t1,
+              (int64_t)b * max_chunks + c, direct, lane & 15, lane >> 4);
+}
+
+// Inclusive prefix sum over the 64 lanes of a wave with DPP moves: a
+// Hillis-Steele scan inside each row of 16 lanes (a lane without a source in
+// its row adds 0), then the last lane of row 0 / row 2 is added to rows 1 / 3
+// (row_bcast:15) and the last lane of row 1 to rows 2 and 3 (row_bcast:31).
+__device__ __forceinline__ int wave_inclusive_scan(int x) {
+  x += __builtin_amdgcn_update_dpp(0, x, 0x111, 0xF, 0xF, false);  // row_shr:1
+  x += __builtin_amdgcn_update_dpp(0, x, 0x112, 0xF, 0xF, false);  // row_shr:2
+  x += __builtin_amdgcn_update_dpp(0, x, 0x114, 0xF, 0xF, false);  // row_shr:4
+  x += __builtin_amdgcn_update_dpp(0, x, 0x118, 0xF, 0xF, false);  // row_shr:8
+  x += __builtin_amdgcn_update_dpp(0, x, 0x142, 0xA, 0xF, false);  // row_bcast:15 -> rows 1, 3
+  x += __builtin_amdgcn_update_dpp(0, x, 0x143, 0xC, 0xF, false);  // row_bcast:31 -> rows 2, 3
+  return x;
+}
+
+// Balanced split: the 32-position steps of all sequences, laid end to end in
+// batch order, are cut into `num_wgs` equal runs of `S` steps (at least
+// `min_steps`); workgroup g owns steps [g*S, (g+1)*S) whatever sequences they
+// belong to.  A run that crosses a sequence boundary is processed as one
+// segment per sequence.  The segment of (workgroup g, sequence b) uses partial
+// slot g + b, which is unique because g and b only grow along the runs; the
+// slots of one sequence are consecutive.  Every workgroup derives the cut from
+// context_lens itself (a wave-wide prefix sum over the batch), so the host
+// never needs the lengths.  Workgroup 0 also leaves the exclusive prefix sums
+// (steps before each sequence, total at [batch]) in `prefix` for the combine
+// pass.  grid.x = num_wgs, grid.y = num_kv_heads / NW, block = NW * 64.
+template <int NW>
+__global__ __launch_bounds__(NW * 64) void paged_decode_balanced_kernel(DecodeArgs a, int batch,
+                                                                        int num_wgs,
+                                                                        int min_steps,
+                                                                        int32_t* prefix) {
+  __shared__ uint4 k_tile[NW][kStep * kLdsRowPieces];
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int lane = threadIdx.x & 63;
+  const int g = blockIdx.x;
+  const int cap = a.max_blocks * a.block_size;
+  const bool writer = g == 0 && blockIdx.y == 0 && wave == 0;
+
+  auto ctx_of = [&](int idx) { return idx < batch ? min(max(a.context_lens[idx], 0), cap) : 0; };
+  auto steps_of = [&](int idx) { return (ctx_of(idx) + kStep - 1) / kStep; };
+
+  // One pass over the batch, 64 sequences at a time: total number of steps,
+  // and for the first kKeep groups the per-lane (steps, steps before) pairs are
+  // kept so that locating the start below needs no second read.
+  constexpr int kKeep = 4;
+  int kept_ctx[kKeep], kept_excl[kKeep];
+#pragma unroll
+  for (int k = 0; k < kKeep; ++k) kept_ctx[k] = kept_excl[k] = 0;
+  int total = 0, total_kept = 0;
+#pragma unroll
+  for (int k = 0; k < kKeep; ++k) {
+    if (k * 64 < batch) {
+      kept_ctx[k] = ctx_of(k * 64 + lane);
+      const int n = (kept_ctx[k] + kStep - 1) / kStep;
+      const int incl = wave_inclusive_scan(n);
+      kept_excl[k] = total + incl - n;
+      if (writer && k * 64 + lane < batch) prefix[k * 64 + lane] = kept_excl[k];
+      total += __builtin_amdgcn_readlane(incl, 63);
+    }
+  }
+  total_kept = total;
+  for (int base = kKeep * 64; base < batch; base += 64) {
+    const int n = steps_of(base + lane);
+    const int incl = wave_inclusive_scan(n);
+    if (writer && base + lane < batch) prefix[base + lane] = total + incl - n;
+    total += __builtin_amdgcn_readlane(incl, 63);
+  }
+  if (writer && lane == 0) prefix[batch] = total;
+  const int run = max((total + num_wgs - 1) / num_wgs, min_steps);
+  const int start = g * run;
+  if (start >= total) return;
+  const int end = min(total, start + run);
+
+  // the sequence that holds step `start`, the steps before it and its length
+  int b = batch, before = total, first_ctx = -1;
+  bool found = false;
+#pragma unroll
+  for (int k = 0; k < kKeep; ++k) {
+    const int n = (kept_ctx[k] + kStep - 1) / kStep;
+    const unsigned long long hit =
+        __ballot(!found && n > 0 && kept_excl[k] <= start && start < kept_excl[k] + n);
+    if (hit != 0ull) {
+      const int src = __builtin_ctzll(hit);
+      b = k * 64 + src;
+      before = __shfl(kept_excl[k], src, 64);
+      first_ctx = __shfl(kept_ctx[k], src, 64);
+      found = true;
+    }
+  }
+  if (!found) {
+    int running = total_kept;
+    for (int base = kKeep * 64; base < batch; base += 64) {
+      const int n = steps_of(base + lane);
+      const int incl = wave_inclusive_scan(n);
+      const int excl = running + incl - n;
+      const unsigned long long hit = __ballot(n > 0 && excl <= start && start < excl + n);
+      if (hit != 0ull) {
+        const int src = __builtin_ctzll(hit);
+        b = base + src;
+        before = __shfl(excl, src, 64);
+        break;
+      }
+      running += __builtin_amdgcn_readlane(incl, 63);
+    }
+  }
+  b = __builtin_amdgcn_readfirstlane(b);
+  before = __builtin_amdgcn_readfirstlane(before);
+  first_ctx = __builtin_amdgcn_readfirstlane(first_ctx);
+
+  // Walk the run.  The guards (b inside the batch, pos not before the
+  // sequence) cannot fire when the prefix sums are right; they keep every
+  // index in range regardless.
+  // Every quantity of the walk is wave-uniform; readfirstlane says so, so
+  // that lengths, page lookups and address arithmetic stay on the scalar unit.
+  int pos = start;
+  while (pos < end && b < batch && pos >= before) {
+    const int sb = __builtin_amdgcn_readfirstlane(b);
+    // the first sequence's length is already in registers from the scan
+    const int ctx = __builtin_amdgcn_readfirstlane(
+        first_ctx >= 0 ? first_ctx : min(max(as_constant(a.context_lens)[sb], 0), cap));
+    first_ctx = -1;
+    const int nb = (ctx + kStep - 1) / kStep;
+    if (pos >= before + nb) {  // empty sequence, or this one is finished
+      before += nb;
+      b = sb + 1;
+      continue;
+    }
+    const int seg_end = min(end, before + nb);
+    const int t0 = __builtin_amdgcn_readfirstlane((pos - before) * kStep);
+    const int t1 = __builtin_amdgcn_readfirstlane(min(ctx, (seg_end - before) * kStep));
+    const bool direct = pos == before && seg_end == before + nb;
+    run_segment(a, k_tile[wave], sb, blockIdx.y * NW + wave, t0, t1, (int64_t)(g + sb), direct,
+                lane & 15, lane >> 4);
+    pos = seg_end;
+  }
+}
+
+// Merge the partials of one (sequence, query head).  grid = (B, Hq), block = 128
+// lanes, one per output dim.  Fixed-chunk mode (prefix == nullptr): the
+// partials of sequence b are slots b*max_chunks .. + ceil(ctx/chunk).  Balanced
+// mode: they are slots g_first + b .. g_last + b, where g_first..g_last are the
+// workgroups whose runs of `run` steps touch the sequence.  A sequence with one
+// partial was written by the split kernel itself; an empty one gives zeros.
 __global__ __launch_bounds__(kHeadDim) void paged_decode_combine_kernel(
     const float* __restrict__ part_o, const float* __restrict__ part_ml,
-    const int32_t* __restrict__ context_lens, uint16_t* __restrict__ out, int num_heads,
-    int chunk, int max_chunks, int max_positions, float scale_log2e) {
+    const int32_t* __restrict__ context_lens, const int32_t* __restrict__ prefix,
+    uint16_t* __restrict__ out, int num_heads, int chunk, int max_chunks, int max_positions,
+    int batch, int num_wgs, int min_steps, float scale_log2e) {
   const int b = blockIdx.x, h = blockIdx.y, d = threadIdx.x;
-  const int ctx = min(context_lens[b], max_positions);
-  const int nchunks = ctx <= 0 ? 0 : (ctx + chunk - 1) / chunk;
-  if (nchunks == 1) return;  // written by the split-K kernel itself
+  int nparts;
+  int64_t first;
+  if (prefix == nullptr) {
+    const int ctx = min(context_lens[b], max_positions);
+    nparts = ctx <= 0 ? 0 : (ctx + chunk - 1) / chunk;
+    first = (int64_t)b * max_chunks;
+  } else {
+    const int before = prefix[b], nb = prefix[b + 1] - before, total = prefix[batch];
+    const int run = max((total + num_wgs - 1) / num_wgs, min_steps);
+    const int g_first = before / run;
+    nparts = nb <= 0 ? 0 : (before + nb - 1) / run - g_first + 1;
+    first = (int64_t)g_first + b;
+  }
+  if (nparts == 1) return;  // written by the split kernel itself
   uint16_t* o = out + ((int64_t)b * num_heads + h) * kHeadDim + d;
-  if (nchunks == 0) {  // empty sequence: 0 / (0 + 1e-9)
+  if (nparts == 0) {  // empty sequence: 0 / (0 + 1e-9)
     *o = 0;
     return;
   }
-  const int64_t base = (int64_t)b * max_chunks * num_heads + h;
+  const int64_t base = first * num_heads + h;
   const float2* ml = reinterpret_cast<const float2*>(part_ml);
-  float m = kNegBig;
-  for (int c = 0; c < nchunks; ++c) m = fmaxf(m, ml[base + (int64_t)c * num_heads].x);
-  float num = 0.f, den = 0.f;
-  for (int c = 0; c < nchunks; ++c) {
-    const int64_t slot = base + (int64_t)c * num_heads;
-    const float2 v = ml[slot];
-    const float w = __builtin_amdgcn_exp2f((v.x - m) * scale_log2e);
-    den = fmaf(w, v.y, den);
-    num = fmaf(w, part_o[slot * kHeadDim + d], num);
+  // One pass, 8 partials at a time with all their loads issued together, merged
+  // with the running-max rescale.
+  float m = kNegBig, num = 0.f, den = 0.f;
+  for (int c0 = 0; c0 < nparts; c0 += 8) {
+    float2 mlv[8];
+    float po[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      const int64_t row = base + (int64_t)min(c0 + i, nparts - 1) * num_heads;
+      mlv[i] = ml[row];
+      po[i] = part_o[row * kHeadDim + d];
+    }
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      if (c0 + i < nparts) {
+        const float m_new = fmaxf(m, mlv[i].x);
+        const float keep = __builtin_amdgcn_exp2f((m - m_new) * scale_log2e);
+        const float w = __builtin_amdgcn_exp2f((mlv[i].x - m_new) * scale_log2e);
+        num = fmaf(num, keep, w * po[i]);
+        den = fmaf(den, keep, w * mlv[i].y);
+        m = m_new;
+      }
+    }
   }
   const float res = num / (den + 1e-9f);
   *o = (uint16_t)(pack_bf16x2(res, 0.f) & 0xFFFFu);
@@ -331,18 +535,55 @@ __global__ __launch_bounds__(kHeadDim) void paged_decode_combine_kernel(
 
 int round_up(int x, int m) { return (x + m - 1) / m * m; }
 
+// Balanced mode launches at most one workgroup per CU of an MI355X, and never
+// gives a workgroup fewer than 4 steps (128 positions): below that the
+// partials cost more than the split gains.
+constexpr int kMaxBalancedWorkgroups = 256;
+constexpr int kMinBalancedSteps = 4;
+
+int balanced_workgroups(int64_t batch, int64_t max_blocks, int64_t block_size) {
+  const int64_t max_steps = batch * ((max_blocks * block_size + kStep - 1) / kStep);
+  const int64_t wgs = (max_steps + kMinBalancedSteps - 1) / kMinBalancedSteps;
+  return (int)(wgs < 1 ? 1 : wgs > kMaxBalancedWorkgroups ? kMaxBalancedWorkgroups : wgs);
+}
+
+// Workspace layout.  Fixed chunks: slots = batch * max_chunks.  Balanced:
+// slots = workgroups + batch, followed by the int32 prefix array [batch + 1].
+struct WorkspacePlan {
+  int64_t slots;
+  int max_chunks;   // fixed-chunk mode only
+  int num_wgs;      // balanced mode only
+  size_t bytes;
+};
+
+bool plan_workspace(int64_t batch, int64_t num_heads, int64_t max_blocks, int64_t block_size,
+                    int chunk, WorkspacePlan* plan) {
+  if (chunk == 0) {
+    plan->num_wgs = balanced_workgroups(batch, max_blocks, block_size);
+    plan->max_chunks = 0;
+    plan->slots = plan->num_wgs + batch;
+    const size_t floats = (size_t)plan->slots * num_heads * (kHeadDim + 2);
+    plan->bytes = floats * sizeof(float) + (size_t)(batch + 1) * sizeof(int32_t);
+    return batch * ((max_blocks * block_size + kStep - 1) / kStep) <= INT32_MAX;
+  }
+  const int64_t mc = (max_blocks * block_size + chunk - 1) / chunk;
+  if (batch * mc > INT32_MAX) return false;
+  plan->num_wgs = 0;
+  plan->max_chunks = (int)mc;
+  plan->slots = batch * mc;
+  plan->bytes = (size_t)plan->slots * num_heads * (kHeadDim + 2) * sizeof(float);
+  return true;
+}
+
 }  // namespace
 
 extern "C" int32_t nvj_paged_decode_default_chunk(int32_t batch, int32_t num_kv_heads,
                                                   int32_t max_blocks, int32_t block_size) {
   if (batch <= 0 || num_kv_heads <= 0 || max_blocks <= 0 || block_size <= 0) return 256;
-  // One workgroup (8 waves at ~230 VGPRs) is resident per CU, and the kernel
-  // is fastest when a launch is exactly one workgroup per CU (256 on MI355X):
-  // pick the chunk that gives that when every sequence is at full length, if
-  // it is at most 2048 positions.  Beyond that the launch runs in several
-  // rounds anyway and 1024 keeps ragged batches balanced (a long chunk that
-  // starts late becomes the tail of the whole launch).  Below 128 positions
-  // the partials only add combine work.
+  // One 8-wave workgroup is resident per CU and a launch is fastest at exactly
+  // one workgroup per CU (256 on MI355X): the chunk that gives that when every
+  // sequence is at full length, if it is at most 2048 positions; else 1024,
+  // which keeps ragged batches balanced; never below 128.
   const int64_t positions = (int64_t)batch * max_blocks * block_size;
   int64_t chunk = (positions + 255) / 256;
   if (chunk < 128) chunk = 128;
@@ -350,23 +591,16 @@ extern "C" int32_t nvj_paged_decode_default_chunk(int32_t batch, int32_t num_kv_
   return round_up((int)chunk, kStep);
 }
 
-static int resolve_chunk(int32_t batch, int32_t num_kv_heads, int32_t max_blocks,
-                         int32_t block_size, int32_t chunk) {
-  if (chunk == 0) chunk = nvj_paged_decode_default_chunk(batch, num_kv_heads, max_blocks, block_size);
-  return chunk;
-}
-
 extern "C" size_t nvj_paged_decode_workspace_bytes(int32_t batch, int32_t num_heads,
                                                    int32_t head_dim, int32_t max_blocks,
                                                    int32_t block_size, int32_t num_kv_heads,
                                                    int32_t chunk) {
-  if (batch <= 0 || num_heads <= 0 || head_dim <= 0 || max_blocks <= 0 || block_size <= 0 ||
-      chunk < 0 || chunk % kStep != 0)
+  if (batch <= 0 || num_heads <= 0 || head_dim != kHeadDim || max_blocks <= 0 ||
+      block_size <= 0 || num_kv_heads <= 0 || chunk < 0 || chunk % kStep != 0)
     return 0;
-  chunk = resolve_chunk(batch, num_kv_heads, max_blocks, block_size, chunk);
-  const int64_t max_chunks = ((int64_t)max_blocks * block_size + chunk - 1) / chunk;
-  const int64_t slots = (int64_t)batch * max_chunks * num_heads;
-  return (size_t)(slots * (head_dim + 2) * sizeof(float));
+  WorkspacePlan plan;
+  if (!plan_workspace(batch, num_heads, max_blocks, block_size, chunk, &plan)) return 0;
+  return plan.bytes;
 }
 
 extern "C" int nvj_paged_decode_launch_phases(void* stream, const void* q, const void* k_cache,
@@ -385,6 +619,7 @@ extern "C" int nvj_paged_decode_launch_phases(void* stream, const void* q, const
   const int group = num_heads / num_kv_heads;
   if (head_dim != kHeadDim || group > 16 || block_size % kStep != 0 || chunk % kStep != 0)
     return NVJ_ERR_UNSUPPORTED;
+  if ((int64_t)max_blocks * block_size > INT32_MAX) return NVJ_ERR_BAD_SHAPE;
   if (batch == 0) return NVJ_OK;
   if (!q || !k_cache || !v_cache || !context_lens || !out) return NVJ_ERR_NULL_POINTER;
   if (max_blocks > 0 && !block_tables) return NVJ_ERR_NULL_POINTER;
@@ -393,40 +628,62 @@ extern "C" int nvj_paged_decode_launch_phases(void* stream, const void* q, const
        reinterpret_cast<uintptr_t>(workspace)) & 15u)
     return NVJ_ERR_WORKSPACE;
   hipStream_t s = static_cast<hipStream_t>(stream);
-  const float scale_log2e = scale * kLog2e;
 
-  int max_chunks = 1;
-  float* part_o = nullptr;
-  float* part_ml = nullptr;
+  DecodeArgs a;
+  a.q = static_cast<const uint4*>(q);
+  a.k_cache = static_cast<const char*>(k_cache);
+  a.v_cache = static_cast<const char*>(v_cache);
+  a.block_tables = block_tables;
+  a.context_lens = context_lens;
+  a.out = static_cast<uint4*>(out);
+  a.part_o = nullptr;
+  a.part_ml = nullptr;
+  a.num_heads = num_heads;
+  a.num_kv_heads = num_kv_heads;
+  a.group = group;
+  a.block_size = block_size;
+  a.max_blocks = max_blocks;
+  a.num_blocks = num_blocks;
+  a.scale_log2e = scale * kLog2e;
+
+  WorkspacePlan plan = {0, 1, 0, 0};
+  int32_t* prefix = nullptr;
   if (max_blocks > 0) {
-    chunk = resolve_chunk(batch, num_kv_heads, max_blocks, block_size, chunk);
-    const int64_t mc = ((int64_t)max_blocks * block_size + chunk - 1) / chunk;
-    const int64_t slots = (int64_t)batch * mc * num_heads;
-    if ((int64_t)batch * mc > INT32_MAX) return NVJ_ERR_BAD_SHAPE;
-    const size_t need = (size_t)slots * (kHeadDim + 2) * sizeof(float);
-    if (!workspace || workspace_bytes < need) return NVJ_ERR_WORKSPACE;
-    max_chunks = (int)mc;
-    part_o = static_cast<float*>(workspace);
-    part_ml = part_o + slots * kHeadDim;
+    if (!plan_workspace(batch, num_heads, max_blocks, block_size, chunk, &plan))
+      return NVJ_ERR_BAD_SHAPE;
+    if (!workspace || workspace_bytes < plan.bytes) return NVJ_ERR_WORKSPACE;
+    a.part_o = static_cast<float*>(workspace);
+    a.part_ml = a.part_o + plan.slots * num_heads * kHeadDim;
+    if (chunk == 0) prefix = reinterpret_cast<int32_t*>(a.part_ml + plan.slots * num_heads * 2);
 
-    const int nw = num_kv_heads % 8 == 0 ? 8 : num_kv_heads % 4 == 0 ? 4 : num_kv_heads % 2 == 0 ? 2 : 1;
-    dim3 grid((unsigned)(batch * max_chunks), (unsigned)(num_kv_heads / nw));
-    const uint4* q4 = static_cast<const uint4*>(q);
-    const char* k4 = static_cast<const char*>(k_cache);
-    const char* v4 = static_cast<const char*>(v_cache);
-    uint4* o4 = static_cast<uint4*>(out);
     if (phases & NVJ_PHASE_SPLITK) {
-#define NVJ_LAUNCH_SPLITK(NWV)                                                               \
-  paged_decode_splitk_kernel<NWV><<<grid, dim3(NWV * 64), 0, s>>>(                           \
-      q4, k4, v4, block_tables, context_lens, o4, part_o, part_ml, num_heads, num_kv_heads,  \
-      group, block_size, max_blocks, num_blocks, chunk, max_chunks, scale_log2e)
-    switch (nw) {
-      case 8: NVJ_LAUNCH_SPLITK(8); break;
-      case 4: NVJ_LAUNCH_SPLITK(4); break;
-      case 2: NVJ_LAUNCH_SPLITK(2); break;
-      default: NVJ_LAUNCH_SPLITK(1); break;
-    }
-#undef NVJ_LAUNCH_SPLITK
+      const int nw =
+          num_kv_heads % 8 == 0 ? 8 : num_kv_heads % 4 == 0 ? 4 : num_kv_heads % 2 == 0 ? 2 : 1;
+      const unsigned gy = (unsigned)(num_kv_heads / nw);
+      if (chunk == 0) {
+        const dim3 grid((unsigned)plan.num_wgs, gy);
+#define NVJ_LAUNCH(NWV)                                               \
+  paged_decode_balanced_kernel<NWV><<<grid, dim3(NWV * 64), 0, s>>>( \
+      a, batch, plan.num_wgs, kMinBalancedSteps, prefix)
+        switch (nw) {
+          case 8: NVJ_LAUNCH(8); break;
+          case 4: NVJ_LAUNCH(4); break;
+          case 2: NVJ_LAUNCH(2); break;
+          default: NVJ_LAUNCH(1); break;
+        }
+#undef NVJ_LAUNCH
+      } else {
+        const dim3 grid((unsigned)(batch * plan.max_chunks), gy);
+#define NVJ_LAUNCH(NWV) \
+  paged_decode_splitk_kernel<NWV><<<grid, dim3(NWV * 64), 0, s>>>(a, chunk, plan.max_chunks)
+        switch (nw) {
+          case 8: NVJ_LAUNCH(8); break;
+          case 4: NVJ_LAUNCH(4); break;
+          case 2: NVJ_LAUNCH(2); break;
+          default: NVJ_LAUNCH(1); break;
+        }
+#undef NVJ_LAUNCH
+      }
       if (hipGetLastError() != hipSuccess) return NVJ_ERR_LAUNCH;
     }
   } else {
@@ -434,8 +691,9 @@ extern "C" int nvj_paged_decode_launch_phases(void* stream, const void* q, const
   }
   if (!(phases & NVJ_PHASE_COMBINE)) return NVJ_OK;
   paged_decode_combine_kernel<<<dim3((unsigned)batch, (unsigned)num_heads), dim3(kHeadDim), 0, s>>>(
-      part_o, part_ml, context_lens, static_cast<uint16_t*>(out), num_heads, chunk, max_chunks,
-      max_blocks * block_size, scale_log2e);
+      a.part_o, a.part_ml, context_lens, prefix, static_cast<uint16_t*>(out), num_heads, chunk,
+      plan.max_chunks, max_blocks * block_size, batch, plan.num_wgs, kMinBalancedSteps,
+      a.scale_log2e);
   return hipGetLastError() == hipSuccess ? NVJ_OK : NVJ_ERR_LAUNCH;
 }
 

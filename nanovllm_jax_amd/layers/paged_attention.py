@@ -31,7 +31,8 @@ def _check_device_tensor(t: torch.Tensor, name: str, dtype: torch.dtype, ndim: i
 
 
 def default_chunk(batch: int, num_kv_heads: int, max_blocks: int, block_size: int) -> int:
-    """Positions per workgroup the library picks when ``chunk=0``."""
+    """Fixed chunk (positions per workgroup) the library recommends when a
+    fixed split is wanted; ``chunk=0`` itself selects the balanced split."""
     return int(_lib.load().nvj_paged_decode_default_chunk(batch, num_kv_heads,
                                                           max_blocks, block_size))
 
@@ -58,8 +59,9 @@ def paged_attention(q, k_cache, v_cache, block_tables, context_lens, scale, bloc
     scale        softmax scale (Python float)
     block_size   positions per page; must equal ``k_cache.shape[1]``
 
-    Returns [batch, num_heads, head_dim] bf16.  ``chunk`` (positions per
-    workgroup, multiple of 32, 0 = library default), ``out`` and ``workspace``
+    Returns [batch, num_heads, head_dim] bf16.  ``chunk`` (0 = balanced split
+    derived from ``context_lens`` on the device; > 0 = that many positions per
+    workgroup, multiple of 32), ``out`` and ``workspace``
     (uint8 tensor of at least ``paged_decode_workspace_bytes`` bytes) are
     optional tuning/reuse knobs the reference does not have; ``phases`` selects
     the split-K launch, the combine launch or both (timing aid).

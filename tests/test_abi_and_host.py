@@ -71,8 +71,11 @@ def test_workspace_and_chunk_queries():
     need = paged_decode_workspace_bytes(64, 32, 128, 16, 256, 8, 256)
     assert need == 64 * 16 * 32 * (128 + 2) * 4
     assert paged_decode_workspace_bytes(64, 32, 128, 16, 256, 8, 100) == 0   # bad chunk
+    # balanced split: one partial slot per workgroup (<= 256) plus one per sequence,
+    # then batch + 1 prefix sums
     assert paged_decode_workspace_bytes(64, 32, 128, 16, 256, 8, 0) == \
-        paged_decode_workspace_bytes(64, 32, 128, 16, 256, 8, c)
+        (256 + 64) * 32 * (128 + 2) * 4 + 65 * 4
+    assert paged_decode_workspace_bytes(2, 8, 128, 1, 32, 8, 0) == (1 + 2) * 8 * 130 * 4 + 3 * 4
 
 
 def test_host_mirror_refuses_cpu_tensors():

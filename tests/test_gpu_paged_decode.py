@@ -131,3 +131,40 @@ def test_reference_smoke_shape_b64():
     got = run_hip(q, kc, vc, bt, ctx, scale, bs)
     want = oracle(q, kc, vc, bt, ctx, scale, bs)
     assert_close_bf16(got, want, what="reference smoke shape")
+
+
+@pytest.mark.parametrize("B,seed", [(70, 1), (300, 2), (517, 3)])
+def test_balanced_split_many_ragged_sequences(B, seed):
+    """The balanced split (chunk=0) derives its cut from context_lens on the
+    device: exercise runs that span many short sequences, empty sequences in
+    between, batches beyond the 256 sequences whose prefix sums are kept in
+    registers, and compare with a fixed split and the oracle."""
+    print(f"case balanced ragged B={B}", flush=True)
+    rng = np.random.Generator(np.random.PCG64(seed))
+    Hq, Hkv, D, bs = 16, 8, 128, 32
+    ctx = rng.integers(0, 200, size=B)
+    ctx[rng.integers(0, B, size=B // 7)] = 0            # empty sequences
+    ctx[rng.integers(0, B, size=3)] = rng.integers(900, 1500, size=3)   # a few long ones
+    ctx[-1] = 0 if seed == 2 else 777                   # last sequence empty / long
+    NB = int((-(-ctx // bs)).sum()) + 3
+    q, kc, vc, bt, ctx = make_problem(100 + seed, B, Hq, Hkv, D, bs, NB, ctx)
+    scale = 1.0 / np.sqrt(D)
+    want = oracle(q, kc, vc, bt, ctx, scale, bs)
+    got = run_hip(q, kc, vc, bt, ctx, scale, bs, 0)
+    assert_close_bf16(got, want, what=f"balanced B={B}")
+    assert not got[ctx == 0].any()
+    fixed = run_hip(q, kc, vc, bt, ctx, scale, bs, 64)
+    assert_close_bf16(fixed, want, what=f"fixed chunk B={B}")
+
+
+def test_balanced_split_all_empty_and_single_position():
+    print("case balanced all-empty / single position", flush=True)
+    B, Hq, Hkv, D, bs, NB = 9, 32, 8, 128, 256, 12
+    q, kc, vc, bt, ctx = make_problem(5, B, Hq, Hkv, D, bs, NB, [0] * B)
+    got = run_hip(q, kc, vc, bt, ctx, 0.1, bs, 0)
+    assert not got.any()
+    ctx2 = np.zeros(B, np.int32); ctx2[4] = 1
+    q, kc, vc, bt, ctx2 = make_problem(6, B, Hq, Hkv, D, bs, NB, ctx2)
+    got = run_hip(q, kc, vc, bt, ctx2, 0.1, bs, 0)
+    assert np.array_equal(got[4], np.repeat(vc[bt[4, 0], 0], Hq // Hkv, axis=0))
+    assert not np.delete(got, 4, axis=0).any()
