@@ -4,11 +4,13 @@
 // (layers/pallas_attention.py:465-507, :146-238 of the reference) and for the
 // gather + dot_product_attention fallback (layers/attention.py:399-434).
 //
-// Work split.  One workgroup handles `chunk` consecutive positions of one
-// sequence for NW KV heads at once, one wave per KV head, so the workgroup as
-// a whole streams whole 2 KiB cache rows (all heads of a position are
-// contiguous in the [page, position, head, dim] layout).  A wave owns the G
-// query heads of its KV head, so every K/V byte is fetched once per group.
+// Work split.  A workgroup handles a run of positions for NW KV heads at once,
+// one wave per KV head, so the workgroup as a whole streams whole 2 KiB cache
+// rows (all heads of a position are contiguous in the [page, position, head,
+// dim] layout).  A wave owns the G query heads of its KV head, so every K/V
+// byte is fetched once per group.  The runs are either equal cuts of all the
+// steps of the batch, derived on the device from context_lens (balanced split,
+// the default), or fixed chunks of each sequence.
 //
 // Inner step = 32 positions of one page:
 //   * K: 8 x 16-byte loads per lane, quarter-wave = one 256-byte (position,
@@ -24,9 +26,9 @@
 //   * O^T[dim, qhead] += V^T . P^T with 8 MFMAs.
 // Loads for step i+1 are issued before the arithmetic of step i.
 //
-// The partial (unnormalised O, running max, running sum) of every chunk goes
-// to the workspace; the combine kernel merges the chunks of a sequence.  A
-// sequence that fits one chunk is written directly.
+// The partial (unnormalised O, running max, running sum) of every segment goes
+// to the workspace; the combine kernel merges the segments of a sequence.  A
+// sequence that is one segment is written directly.
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
