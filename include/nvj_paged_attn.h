@@ -195,6 +195,34 @@ NVJ_API int nvj_qk_norm_rope_store_launch(void* stream,
                             void* q_out, int32_t num_tokens, int32_t num_heads,
                             int32_t num_kv_heads, int32_t head_dim, int64_t num_slots);
 
+/*
+ * Advance the device-resident metadata of a decode batch by one step, in
+ * place.  Replaces the per-step host rebuild and upload of
+ * ModelRunner._prepare_decode (engine/model_runner.py:334-376): once a step has
+ * produced next_tokens[i] for every sequence, sequence i grows by that token and
+ *
+ *   input_ids[i]    = next_tokens[i]                         (seq.last_token)
+ *   positions[i]    = len - 1
+ *   context_lens[i] = len                                    (len = old length + 1)
+ *   slot_mapping[i] = block_tables[i, (len-1) / block_size] * block_size
+ *                     + (len-1) % block_size
+ *                     (= block_table[-1] * block_size + last_block_num_tokens - 1)
+ *
+ * next_tokens is int32 (token_bytes 4) or int64 (token_bytes 8); all other
+ * arrays are int32 [batch], block_tables int32 [batch, max_blocks].  The host
+ * keeps block_tables current: when a sequence is about to enter a new page the
+ * page number must be in its row before this call (the reference allocates it
+ * in BlockManager.may_append, engine/block_manager.py:215-243).  A row with
+ * context_lens <= 0 is inactive and stays so; a row whose next page is missing
+ * (-1 padding or beyond max_blocks) is left unchanged; both get slot -1, i.e.
+ * their K/V are not stored.
+ */
+NVJ_API int nvj_advance_decode_launch(void* stream, const void* next_tokens,
+                            int32_t token_bytes, int32_t* input_ids, int32_t* positions,
+                            int32_t* context_lens, int32_t* slot_mapping,
+                            const int32_t* block_tables, int32_t batch, int32_t max_blocks,
+                            int32_t block_size);
+
 #ifdef __cplusplus
 }  /* extern "C" */
 #endif

@@ -41,6 +41,9 @@ SYMBOLS = {
         _c.c_void_p, _c.c_void_p, _c.c_int64, _c.c_void_p, _c.c_void_p, _c.c_int32, _c.c_void_p,
         _c.c_void_p, _c.c_float, _c.c_void_p, _c.c_void_p, _c.c_void_p, _c.c_void_p,
         _c.c_int32, _c.c_int32, _c.c_int32, _c.c_int32, _c.c_int64]),
+    "nvj_advance_decode_launch": (_c.c_int, [
+        _c.c_void_p, _c.c_void_p, _c.c_int32, _c.c_void_p, _c.c_void_p, _c.c_void_p, _c.c_void_p,
+        _c.c_void_p, _c.c_int32, _c.c_int32, _c.c_int32]),
 }
 NVJ_PHASE_SPLITK = 1
 NVJ_PHASE_COMBINE = 2

@@ -24,12 +24,14 @@ import numpy as np
 import torch
 import torch.nn.functional as F
 
+from .. import _lib
 from ..layers.attention import Attention
 from ..layers.paged_attention import paged_attention, paged_decode_workspace_bytes
 from ..layers.qk_rope_store import qk_norm_rope_store
 from ..utils.context import AttentionContext, create_decode_context
 
-__all__ = ["DecodeModelConfig", "DecodeStepRunner", "prepare_block_tables", "prepare_decode"]
+__all__ = ["DecodeModelConfig", "DecodeStepRunner", "prepare_block_tables", "prepare_decode",
+           "advance_decode"]
 
 
 @dataclass
@@ -73,6 +75,42 @@ def prepare_decode(last_tokens, seq_lens, block_tables, block_size):
         last_block_tokens = length - (len(table) - 1) * block_size
         slot_mapping[i] = table[-1] * block_size + last_block_tokens - 1
     return input_ids, positions, context_lens, slot_mapping, prepare_block_tables(block_tables)
+
+
+def advance_decode(next_tokens, input_ids, positions, context: AttentionContext, block_size):
+    """Advance the device-resident metadata of a decode batch by one step, in
+    place: every active sequence grows by its ``next_tokens`` entry and
+    ``input_ids / positions / context.context_lens / context.slot_mapping`` get
+    the values ``prepare_decode`` would compute for the grown sequences
+    (``engine/model_runner.py:334-376``), without a host round trip.
+    ``context.block_tables`` must already hold the page a sequence is about to
+    enter."""
+    lib = _lib.load()
+    bt = context.block_tables
+    for name, t in (("next_tokens", next_tokens), ("input_ids", input_ids),
+                    ("positions", positions), ("context_lens", context.context_lens),
+                    ("slot_mapping", context.slot_mapping), ("block_tables", bt)):
+        if not (isinstance(t, torch.Tensor) and t.is_cuda and t.is_contiguous()):
+            raise ValueError(f"{name} must be a contiguous GPU tensor")
+        if name != "next_tokens" and t.dtype != torch.int32:
+            raise ValueError(f"{name} must be int32, got {t.dtype}")
+    if next_tokens.dtype not in (torch.int32, torch.int64):
+        raise ValueError("next_tokens must be int32 or int64")
+    batch = input_ids.shape[0]
+    for name, t in (("next_tokens", next_tokens), ("positions", positions),
+                    ("context_lens", context.context_lens),
+                    ("slot_mapping", context.slot_mapping)):
+        if t.shape != (batch,):
+            raise ValueError(f"{name} must have shape [{batch}]")
+    if bt.dim() != 2 or bt.shape[0] != batch:
+        raise ValueError("block_tables must be [batch, max_blocks]")
+    with torch.cuda.device(input_ids.device):
+        stream = torch.cuda.current_stream(input_ids.device).cuda_stream
+        code = lib.nvj_advance_decode_launch(
+            stream, next_tokens.data_ptr(), next_tokens.element_size(), input_ids.data_ptr(),
+            positions.data_ptr(), context.context_lens.data_ptr(),
+            context.slot_mapping.data_ptr(), bt.data_ptr(), batch, bt.shape[1], int(block_size))
+    _lib.check(code, "nvj_advance_decode_launch")
 
 
 class DecodeStepRunner:
@@ -221,6 +259,38 @@ class DecodeStepRunner:
         graph = torch.cuda.CUDAGraph()
         with torch.cuda.graph(graph):
             out = self.step(input_ids, positions, context)
+        self._graph = graph
+
+        def replay():
+            graph.replay()
+            return out
+        return replay
+
+    def capture_generation(self, input_ids, positions, context):
+        """Capture step + metadata advance in one HIP graph: every replay decodes
+        one token per sequence and leaves ``input_ids / positions / context``
+        ready for the next replay, with nothing but block-table maintenance left
+        to the host.  Returns ``replay() -> token ids of that step``."""
+        c = self.cfg
+        batch, max_blocks = context.block_tables.shape
+        ws = torch.empty(paged_decode_workspace_bytes(batch, c.num_heads, c.head_dim, max_blocks,
+                                                      c.block_size, c.num_kv_heads, 0),
+                         dtype=torch.uint8, device=self.device)
+        for a in self.attn:
+            a.workspace = ws
+        # warm every library handle on a side stream; the warm-up step writes
+        # the K/V rows of the current step, which the captured step rewrites
+        # with the same values, and does not touch the metadata
+        s = torch.cuda.Stream(self.device)
+        s.wait_stream(torch.cuda.current_stream(self.device))
+        with torch.cuda.stream(s):
+            self.step(input_ids, positions, context)
+        torch.cuda.current_stream(self.device).wait_stream(s)
+        torch.cuda.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            out = self.step(input_ids, positions, context)
+            advance_decode(out, input_ids, positions, context, c.block_size)
         self._graph = graph
 
         def replay():

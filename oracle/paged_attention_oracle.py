@@ -56,6 +56,8 @@ __all__ = [
     "build_cos_sin_cache_ref",
     "qk_norm_rope_ref",
     "qk_norm_rope_store_ref",
+    "prepare_decode_ref",
+    "advance_decode_ref",
 ]
 
 
@@ -387,3 +389,64 @@ def qk_norm_rope_store_ref(qkv, positions, cos_sin_cache, q_weight, k_weight, ep
     kc, vc = store_kv_to_cache_ref(k_rot, np.ascontiguousarray(v), k_cache, v_cache,
                                    slot_mapping, negative_slots=negative_slots)
     return f32_to_bf16_bits(q_rot), kc, vc
+
+
+# ---------------------------------------------------------------------------
+# Decode metadata: the filler of the contract
+# ---------------------------------------------------------------------------
+
+def prepare_decode_ref(last_tokens, seq_lens, block_tables, block_size):
+    """``ModelRunner._prepare_decode`` + ``_prepare_block_tables``
+    (``engine/model_runner.py:334-376, 225-246``) for sequences given as
+    (last token, length, list of page numbers): per sequence
+    ``input_ids = last_token``, ``positions = len - 1``, ``context_lens = len``,
+    ``slot = block_table[-1] * block_size + last_block_num_tokens - 1`` with
+    ``last_block_num_tokens = len - (num_blocks - 1) * block_size``
+    (``engine/sequence.py``), tables padded with -1 to the longest.  All int32."""
+    n = len(seq_lens)
+    input_ids = np.empty(n, np.int32)
+    positions = np.empty(n, np.int32)
+    context_lens = np.empty(n, np.int32)
+    slot_mapping = np.empty(n, np.int32)
+    width = max(len(t) for t in block_tables)
+    tables = np.full((n, width), -1, np.int32)                     # :240
+    for i in range(n):
+        length, table = int(seq_lens[i]), list(block_tables[i])
+        input_ids[i] = last_tokens[i]                              # :358
+        positions[i] = length - 1                                  # :359
+        context_lens[i] = length                                   # :360
+        last_block_num_tokens = length - (len(table) - 1) * block_size
+        slot_mapping[i] = table[-1] * block_size + last_block_num_tokens - 1   # :361
+        tables[i, :len(table)] = table
+    return input_ids, positions, context_lens, slot_mapping, tables
+
+
+def advance_decode_ref(next_tokens, input_ids, positions, context_lens, slot_mapping,
+                       block_tables, block_size):
+    """What the arrays of ``prepare_decode_ref`` become once every active
+    sequence has appended ``next_tokens[i]`` (``Sequence.append_token``, then the
+    next ``_prepare_decode``), computed from the padded table instead of the
+    Python lists: the page of position ``len - 1`` is column
+    ``(len - 1) // block_size`` of the row.  Rows with ``context_lens <= 0`` are
+    inactive (slot -1, nothing else changes); a row whose next page is missing
+    (-1, or beyond the table) is left as it is with slot -1.  Returns new arrays."""
+    ids = np.array(input_ids, np.int32, copy=True)
+    pos = np.array(positions, np.int32, copy=True)
+    ctx = np.array(context_lens, np.int32, copy=True)
+    slots = np.array(slot_mapping, np.int32, copy=True)
+    bt = np.asarray(block_tables)
+    for i in range(len(ctx)):
+        if ctx[i] <= 0:
+            slots[i] = -1
+            continue
+        length = int(ctx[i]) + 1
+        page_idx = (length - 1) // block_size
+        page = int(bt[i, page_idx]) if page_idx < bt.shape[1] else -1
+        if page < 0:
+            slots[i] = -1
+            continue
+        ids[i] = next_tokens[i]
+        pos[i] = length - 1
+        ctx[i] = length
+        slots[i] = page * block_size + (length - 1) % block_size
+    return ids, pos, ctx, slots

@@ -118,3 +118,71 @@ def test_graph_replays_match_eager_step():
         torch.cuda.synchronize()
         assert torch.equal(toks, eager_tokens), f"replay {i} differs from eager"
         assert torch.equal(again, eager_tokens)
+
+
+def test_advance_decode_matches_oracle_over_many_steps():
+    """Device-resident metadata advance, bit-exact against the oracle, with the
+    host only maintaining the block tables."""
+    print("case advance_decode many steps", flush=True)
+    from nanovllm_jax_amd import create_decode_context
+    from nanovllm_jax_amd.engine.decode_step import advance_decode
+    from oracle.paged_attention_oracle import advance_decode_ref, prepare_decode_ref
+    bs = 32
+    rng = np.random.Generator(np.random.PCG64(4))
+    B = 300
+    lens = rng.integers(1, 200, B).tolist()
+    lens[5] = 64; lens[6] = 65; lens[7] = 63
+    free = list(range(5000))
+    tables = [[free.pop() for _ in range(-(-n // bs))] for n in lens]
+    ids, pos, ctx, slots, bt = prepare_decode_ref(rng.integers(0, 50000, B).tolist(), lens, tables, bs)
+    ctx[11] = 0                                       # an inactive row
+    width = bt.shape[1] + 2
+    bt_host = np.full((B, width), -1, np.int32); bt_host[:, :bt.shape[1]] = bt
+    dev = "cuda:0"
+    t = lambda a: torch.from_numpy(a.copy()).to(dev)
+    d_ids, d_pos = t(ids), t(pos)
+    d_ctx = create_decode_context(t(ctx), t(slots), t(bt_host))
+    for step in range(40):
+        for i in range(B):                            # host keeps the tables current
+            if ctx[i] > 0 and (ctx[i] + 1) % bs == 1 and len(tables[i]) < width - 1:
+                tables[i].append(free.pop()); bt_host[i, len(tables[i]) - 1] = tables[i][-1]
+        d_ctx.block_tables.copy_(torch.from_numpy(bt_host))
+        dtype = np.int64 if step % 2 else np.int32
+        nxt = rng.integers(0, 50000, B).astype(dtype)
+        ids, pos, ctx, slots = advance_decode_ref(nxt, ids, pos, ctx, slots, bt_host, bs)
+        advance_decode(t(nxt), d_ids, d_pos, d_ctx, bs)
+        torch.cuda.synchronize()
+        assert np.array_equal(d_ids.cpu().numpy(), ids), step
+        assert np.array_equal(d_pos.cpu().numpy(), pos), step
+        assert np.array_equal(d_ctx.context_lens.cpu().numpy(), ctx), step
+        assert np.array_equal(d_ctx.slot_mapping.cpu().numpy(), slots), step
+    assert (slots == -1).sum() >= 1 and ctx[11] == 0
+
+
+def test_generation_graph_matches_host_driven_loop():
+    """step + advance captured in one graph and replayed N times == N eager steps
+    whose metadata the host rebuilds each time (the reference's way)."""
+    print("case generation graph vs host loop", flush=True)
+    cfg, dev_runner = _small_runner()
+    _, host_runner = _small_runner()
+    last, lens, tables = _batch(cfg)
+    lens = [5, 250, 100, 700]                          # room inside the last page for 5 steps
+    rng = np.random.Generator(np.random.PCG64(9))
+    pages = rng.permutation(cfg.num_kvcache_blocks).tolist()
+    tables, off = [], 0
+    for n in lens:
+        k = -(-(n + 6) // cfg.block_size)
+        tables.append(pages[off:off + k]); off += k
+    ids, pos, ctx = dev_runner.make_inputs(last, lens, tables)
+    replay = dev_runner.capture_generation(ids, pos, ctx)
+    cur_last, cur_lens = list(last), list(lens)
+    for step in range(5):
+        used = [t[:-(-n // cfg.block_size)] for t, n in zip(tables, cur_lens)]
+        h_ids, h_pos, h_ctx = host_runner.make_inputs(cur_last, cur_lens, used)
+        want = host_runner.step(h_ids, h_pos, h_ctx).cpu()
+        got = replay().cpu()
+        torch.cuda.synchronize()
+        assert torch.equal(got, want), f"step {step}: {got.tolist()} vs {want.tolist()}"
+        cur_last = want.tolist()
+        cur_lens = [n + 1 for n in cur_lens]
+    assert ctx.context_lens.cpu().tolist() == cur_lens

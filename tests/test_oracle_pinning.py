@@ -289,3 +289,49 @@ def test_qk_norm_rope_store_composes_the_pieces():
             assert np.array_equal(k2[s], kr[t]) and np.array_equal(v2[s], vh[t])
     untouched = [i for i in range(16) if i not in (3, 15, 0)]
     assert np.array_equal(k2[untouched], kc[untouched]) and np.array_equal(v2[untouched], vc[untouched])
+
+
+# ---------------------------------------------------------------- decode metadata
+def test_prepare_and_advance_decode_against_a_sequence_simulation():
+    """Brute force: keep Python-side sequences (token list + page list, a new page
+    whenever the length crosses a page boundary, as BlockManager.may_append does)
+    and rebuild the arrays from scratch every step; the in-place advance must give
+    the same arrays."""
+    from nanovllm_jax_amd.engine.decode_step import prepare_decode
+    from oracle.paged_attention_oracle import advance_decode_ref, prepare_decode_ref
+    bs = 4
+    rng = np.random.Generator(np.random.PCG64(8))
+    lens = [1, 3, 4, 5, 8, 11]
+    free = list(range(100, 200))
+    tables = [[free.pop() for _ in range(-(-n // bs))] for n in lens]
+    last = rng.integers(0, 1000, len(lens)).tolist()
+    ids, pos, ctx, slots, bt = prepare_decode_ref(last, lens, tables, bs)
+    # the package's host filler is the same restatement
+    for a, b in zip(prepare_decode(last, lens, tables, bs), (ids, pos, ctx, slots, bt)):
+        assert np.array_equal(a, b)
+    # hand-checked values: length 5, pages [p0, p1] -> slot p1*4 + 0; length 4 -> p0*4 + 3
+    assert slots[3] == tables[3][1] * bs + 0 and slots[2] == tables[2][0] * bs + 3
+    assert list(pos) == [n - 1 for n in lens] and list(ctx) == lens
+    width = 6
+    bt_dev = np.full((len(lens), width), -1, np.int32); bt_dev[:, :bt.shape[1]] = bt
+    for step in range(9):
+        nxt = rng.integers(0, 1000, len(lens))
+        for i in range(len(lens)):                    # sequences append, pages are added on demand
+            lens[i] += 1
+            if lens[i] % bs == 1:
+                tables[i].append(free.pop()); bt_dev[i, len(tables[i]) - 1] = tables[i][-1]
+        want = prepare_decode_ref(nxt.tolist(), lens, tables, bs)
+        ids, pos, ctx, slots = advance_decode_ref(nxt, ids, pos, ctx, slots, bt_dev, bs)
+        assert np.array_equal(ids, want[0]) and np.array_equal(pos, want[1])
+        assert np.array_equal(ctx, want[2]) and np.array_equal(slots, want[3])
+
+
+def test_advance_decode_inactive_and_missing_page():
+    from oracle.paged_attention_oracle import advance_decode_ref
+    bs = 4
+    ids = np.array([7, 8, 9], np.int32); pos = np.array([3, 0, 3], np.int32)
+    ctx = np.array([4, 0, 4], np.int32); slots = np.array([19, 5, 23], np.int32)
+    bt = np.array([[4, -1], [1, 2], [5, 6]], np.int32)
+    i2, p2, c2, s2 = advance_decode_ref([70, 80, 90], ids, pos, ctx, slots, bt, bs)
+    assert list(c2) == [4, 0, 5] and list(s2) == [-1, -1, 24]      # row 0: next page missing
+    assert list(i2) == [7, 8, 90] and list(p2) == [3, 0, 4]
