@@ -56,5 +56,34 @@ def build(verbose: bool = True, extra_flags: tuple[str, ...] = ()) -> str:
     return LIB_PATH
 
 
+def xla_ffi_include_dir() -> str | None:
+    """Directory of the XLA FFI headers (they ship inside jaxlib), or None."""
+    try:
+        import jax.ffi  # noqa: F401  (absent from images without JAX)
+        return jax.ffi.include_dir()
+    except Exception:
+        return None
+
+
+def build_xla_ffi(verbose: bool = True) -> str | None:
+    """Compile the XLA FFI handlers next to the C-ABI library when the XLA FFI
+    headers can be found; otherwise say so and return None."""
+    inc = xla_ffi_include_dir()
+    if inc is None:
+        if verbose:
+            print("[build] XLA FFI headers not found (jax is not installed): "
+                  "csrc/xla_ffi/nvj_xla_ffi.cc skipped", flush=True)
+        return None
+    out = os.path.join(NATIVE_DIR, "libnvj_xla_ffi.so")
+    cmd = [hipcc_path(), "--offload-arch=gfx950", "-O2", "-std=c++17", "-fPIC", "-shared",
+           "-I", inc, "-I", os.path.join(REPO_DIR, "include"),
+           os.path.join(CSRC_DIR, "xla_ffi", "nvj_xla_ffi.cc"),
+           "-L", NATIVE_DIR, "-lnvj_paged_attn", "-Wl,-rpath,$ORIGIN", "-o", out]
+    if verbose:
+        print("[build]", " ".join(cmd), flush=True)
+    subprocess.run(cmd, check=True)
+    return out
+
+
 if __name__ == "__main__":
     print(build(extra_flags=tuple(sys.argv[1:])))
