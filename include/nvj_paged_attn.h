@@ -128,8 +128,9 @@ NVJ_API size_t nvj_paged_decode_workspace_bytes(int32_t batch, int32_t num_heads
  *
  * Two launches on `stream`: the split-K kernel (each workgroup streams its
  * share of positions for all KV heads) and the combine pass.
- * Supported: head_dim 128, num_heads / num_kv_heads <= 16, block_size a
- * multiple of 32, chunk a multiple of 32 (0 = balanced split).
+ * Supported: head_dim 128 (every Qwen3 size) or 64 (the reference's toy test
+ * shapes), num_heads / num_kv_heads <= 16, block_size a multiple of 32, chunk
+ * a multiple of 32 (0 = balanced split).
  */
 NVJ_API int nvj_paged_decode_launch(void* stream,
                             const void* q, const void* k_cache, const void* v_cache,

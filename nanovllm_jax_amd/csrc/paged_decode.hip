@@ -39,10 +39,19 @@ namespace {
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
 typedef __attribute__((ext_vector_type(4))) float f32x4;
 
-constexpr int kHeadDim = 128;
+constexpr int kMaxHeadDim = 128;     // head_dim is a template parameter: 128 or 64
 constexpr int kStep = 32;            // positions per inner step
-constexpr int kRowPieces = 16;       // 16-byte pieces per (position, head) row
-constexpr int kLdsRowPieces = 17;    // padded LDS row, in 16-byte pieces
+// A (position, head) row of D bf16 is D/8 16-byte pieces; the LDS tile pads a
+// row by one piece so that the 16 rows an MFMA operand read touches fall on
+// different banks.
+template <int D> struct HeadDim {
+  static_assert(D == 128 || D == 64, "head_dim 128 or 64");
+  static constexpr int kPieces = D / 8;             // 16 or 8
+  static constexpr int kLdsRowPieces = kPieces + 1;
+  static constexpr int kPosPerLoad = 64 / kPieces;  // positions one 64-lane load covers: 4 or 8
+  static constexpr int kKLoads = kStep / kPosPerLoad;  // K loads per lane per step: 8 or 4
+  static constexpr int kQkSteps = D / 32;           // MFMA reduction steps of Q.K: 4 or 2
+};
 constexpr float kNegBig = -1.0e30f;  // stands for -inf without inf-inf hazards
 constexpr float kLog2e = 1.4426950408889634f;
 
@@ -68,23 +77,28 @@ __device__ __forceinline__ uint4 load_piece(const char* base, uint32_t off) {
   return make_uint4(t[0], t[1], t[2], t[3]);
 }
 
-// K of one step: load slot i of lane (kg, r) is position 4*i + kg, piece r, so
-// a quarter-wave reads one whole 256-byte (position, head) row.  In a full
-// step the position splits into a uniform part (4*i rows, folded into the
-// scalar base) and one per-lane offset shared by all 8 loads; a TAIL step
-// clamps every slot to the last live position so that nothing at or beyond
-// the context length is ever read.
-template <bool TAIL>
-__device__ __forceinline__ void issue_k_loads(uint4 (&kreg)[8], const char* base, int kg,
-                                              int last, uint32_t row_bytes,
-                                              uint32_t lane_bytes) {
+// K of one step: 64 lanes cover kPosPerLoad whole (position, head) rows per
+// load (lane -> position lane / kPieces, piece lane % kPieces), so every group
+// of kPieces lanes reads one contiguous row (a quarter-wave at head_dim 128).
+// In a full step the position splits into a uniform part (folded into the
+// scalar base) and one per-lane offset shared by all loads; a TAIL step clamps
+// every slot to the last live position so that nothing at or beyond the
+// context length is ever read.
+template <bool TAIL, int D>
+__device__ __forceinline__ void issue_k_loads(uint4 (&kreg)[HeadDim<D>::kKLoads],
+                                              const char* base, int lane, int last,
+                                              uint32_t row_bytes) {
+  using H = HeadDim<D>;
+  const int pos_lane = lane / H::kPieces;
+  const uint32_t piece_bytes = (uint32_t)(lane % H::kPieces) * 16u;
 #pragma unroll
-  for (int i = 0; i < 8; ++i) {
+  for (int i = 0; i < H::kKLoads; ++i) {
     if constexpr (TAIL) {
-      kreg[i] = load_piece(base, (uint32_t)min(4 * i + kg, last) * row_bytes + lane_bytes);
+      kreg[i] = load_piece(
+          base, (uint32_t)min(H::kPosPerLoad * i + pos_lane, last) * row_bytes + piece_bytes);
     } else {
-      kreg[i] = load_piece(base + (size_t)(4 * i) * row_bytes,
-                           (uint32_t)kg * row_bytes + lane_bytes);
+      kreg[i] = load_piece(base + (size_t)(H::kPosPerLoad * i) * row_bytes,
+                           (uint32_t)pos_lane * row_bytes + piece_bytes);
     }
   }
 }
@@ -92,14 +106,20 @@ __device__ __forceinline__ void issue_k_loads(uint4 (&kreg)[8], const char* base
 // V of one step: load slot j of lane (kg, r) is the position that reduction
 // slot j of k-group kg stands for in the P^T operand: 4*kg + j from the first
 // S^T tile, 16 + 4*kg + (j - 4) from the second.
-template <bool TAIL>
-__device__ __forceinline__ void issue_v_loads(uint4 (&vreg)[8], const char* base, int kg,
-                                              int last, uint32_t row_bytes,
-                                              uint32_t lane_bytes) {
+template <bool TAIL, int D>
+__device__ __forceinline__ void issue_v_loads(uint4 (&vreg)[8], const char* base, int kg, int r,
+                                              int last, uint32_t row_bytes) {
+  // lane (kg, r) fetches piece r (dims 8r .. 8r+7) of its 8 positions; at
+  // head_dim 64 there are only 8 pieces and lanes r >= 8 hold zeros
+  const bool live = r < HeadDim<D>::kPieces;
+  const uint32_t lane_bytes = (uint32_t)r * 16u;
+  const uint4 zero = make_uint4(0u, 0u, 0u, 0u);
 #pragma unroll
   for (int j = 0; j < 8; ++j) {
     const int uni = (j < 4) ? j : (16 + j - 4);   // uniform part of the position
-    if constexpr (TAIL) {
+    if (!live) {
+      vreg[j] = zero;
+    } else if constexpr (TAIL) {
       vreg[j] = load_piece(base, (uint32_t)min(4 * kg + uni, last) * row_bytes + lane_bytes);
     } else {
       vreg[j] = load_piece(base + (size_t)uni * row_bytes,
@@ -136,9 +156,13 @@ struct DecodeArgs {
 // kvh.  `direct` means the segment is the whole sequence: the normalised bf16
 // result goes straight to `out`; otherwise the unnormalised partial goes to
 // partial slot `slot` of the workspace.  t0 is a multiple of 32, t0 < t1.
+template <int D>
 __device__ __forceinline__ void run_segment(const DecodeArgs& a, uint4* lds, int b, int kvh,
-                                            int t0, int t1, int64_t slot, bool direct, int r,
-                                            int kg) {
+                                            int t0, int t1, int64_t slot, bool direct,
+                                            int lane) {
+  using H = HeadDim<D>;
+  const int r = lane & 15;   // MFMA row/column index inside a 16-wide tile
+  const int kg = lane >> 4;  // MFMA k-group (which 8 of the 32 reduction slots)
   const uint4* __restrict__ q = a.q;
   const char* __restrict__ k_cache = a.k_cache;
   const char* __restrict__ v_cache = a.v_cache;
@@ -147,26 +171,25 @@ __device__ __forceinline__ void run_segment(const DecodeArgs& a, uint4* lds, int
   const float scale_log2e = a.scale_log2e;
   const int nsteps = (t1 - t0 + kStep - 1) / kStep;
 
-  // Q^T as MFMA B operand for the 4 reduction steps over head_dim:
+  // Q^T as MFMA B operand for the D/32 reduction steps over head_dim:
   // lane (column r = query head of the group, k-group kg) holds dims
   // 32*s + 8*kg .. +8.  Columns >= group are zero.
-  bf16x8 qreg[4];
+  bf16x8 qreg[H::kQkSteps];
   {
     // lanes of padding columns read the group's last head (always in range)
     // and then drop it, so the loads stay unconditional 16-byte loads
     const uint4 zero = make_uint4(0u, 0u, 0u, 0u);
     const uint4* qrow =
-        q + ((int64_t)b * num_heads + (int64_t)kvh * group + min(r, group - 1)) * kRowPieces;
+        q + ((int64_t)b * num_heads + (int64_t)kvh * group + min(r, group - 1)) * H::kPieces;
 #pragma unroll
-    for (int s = 0; s < 4; ++s) {
+    for (int s = 0; s < H::kQkSteps; ++s) {
       const uint4 v = qrow[4 * s + kg];
       qreg[s] = as_bf16x8(r < group ? v : zero);
     }
   }
 
-  const uint32_t row_bytes = (uint32_t)a.num_kv_heads * (kHeadDim * 2);  // one position, all heads
-  const uint32_t lane_bytes = (uint32_t)r * 16u;
-  const int64_t head_bytes = (int64_t)kvh * (kHeadDim * 2);
+  const uint32_t row_bytes = (uint32_t)a.num_kv_heads * (D * 2);  // one position, all heads
+  const int64_t head_bytes = (int64_t)kvh * (D * 2);
   const const_i32_ptr table = as_constant(a.block_tables + (int64_t)b * a.max_blocks);
 
   // wave-uniform byte offset of the first position of a step inside the cache
@@ -177,12 +200,12 @@ __device__ __forceinline__ void run_segment(const DecodeArgs& a, uint4* lds, int
     return ((int64_t)phys * block_size + (ts - page * block_size)) * row_bytes + head_bytes;
   };
 
-  uint4 kreg[8], vreg[8];
+  uint4 kreg[H::kKLoads], vreg[8];
   {
     const int64_t off = step_base(0);
     const int last = min(kStep, t1 - t0) - 1;
-    issue_k_loads<true>(kreg, k_cache + off, kg, last, row_bytes, lane_bytes);
-    issue_v_loads<true>(vreg, v_cache + off, kg, last, row_bytes, lane_bytes);
+    issue_k_loads<true, D>(kreg, k_cache + off, lane, last, row_bytes);
+    issue_v_loads<true, D>(vreg, v_cache + off, kg, r, last, row_bytes);
   }
 
   f32x4 acc[8];
@@ -203,20 +226,22 @@ __device__ __forceinline__ void run_segment(const DecodeArgs& a, uint4* lds, int
 
     // ---- K: registers -> LDS (row = position, padded), then next K loads ----
 #pragma unroll
-    for (int i = 0; i < 8; ++i) lds[(4 * i + kg) * kLdsRowPieces + r] = kreg[i];
+    for (int i = 0; i < H::kKLoads; ++i)
+      lds[(H::kPosPerLoad * i + lane / H::kPieces) * H::kLdsRowPieces + lane % H::kPieces] =
+          kreg[i];
     if (more) {
       if (next_last == kStep - 1)
-        issue_k_loads<false>(kreg, k_cache + next_off, kg, next_last, row_bytes, lane_bytes);
+        issue_k_loads<false, D>(kreg, k_cache + next_off, lane, next_last, row_bytes);
       else
-        issue_k_loads<true>(kreg, k_cache + next_off, kg, next_last, row_bytes, lane_bytes);
+        issue_k_loads<true, D>(kreg, k_cache + next_off, lane, next_last, row_bytes);
     }
 
     // ---- S^T = K . Q^T for two 16-position tiles ----
     f32x4 s0 = {0.f, 0.f, 0.f, 0.f}, s1 = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-    for (int s = 0; s < 4; ++s) {
-      const bf16x8 a0 = as_bf16x8(lds[r * kLdsRowPieces + 4 * s + kg]);
-      const bf16x8 a1 = as_bf16x8(lds[(16 + r) * kLdsRowPieces + 4 * s + kg]);
+    for (int s = 0; s < H::kQkSteps; ++s) {
+      const bf16x8 a0 = as_bf16x8(lds[r * H::kLdsRowPieces + 4 * s + kg]);
+      const bf16x8 a1 = as_bf16x8(lds[(16 + r) * H::kLdsRowPieces + 4 * s + kg]);
       s0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a0, qreg[s], s0, 0, 0, 0);
       s1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a1, qreg[s], s1, 0, 0, 0);
     }
@@ -273,9 +298,9 @@ __device__ __forceinline__ void run_segment(const DecodeArgs& a, uint4* lds, int
     }
     if (more) {
       if (next_last == kStep - 1)
-        issue_v_loads<false>(vreg, v_cache + next_off, kg, next_last, row_bytes, lane_bytes);
+        issue_v_loads<false, D>(vreg, v_cache + next_off, kg, r, next_last, row_bytes);
       else
-        issue_v_loads<true>(vreg, v_cache + next_off, kg, next_last, row_bytes, lane_bytes);
+        issue_v_loads<true, D>(vreg, v_cache + next_off, kg, r, next_last, row_bytes);
     }
 
     // ---- O^T = alpha * O^T + V^T . P^T ----
@@ -292,10 +317,12 @@ __device__ __forceinline__ void run_segment(const DecodeArgs& a, uint4* lds, int
 
   if (r >= group) return;
   const int head = kvh * group + r;
-  // acc[jd][e] is O[head][dim = 32*kg + 8*e + jd]
+  // acc[jd][e] is O[head][dim = 32*kg + 8*e + jd]; at head_dim 64 only k-groups
+  // 0 and 1 hold real dims
+  if (32 * kg >= D) return;
   if (direct) {
     const float inv = 1.0f / (l_run + 1e-9f);
-    uint4* orow = a.out + ((int64_t)b * num_heads + head) * kRowPieces + 4 * kg;
+    uint4* orow = a.out + ((int64_t)b * num_heads + head) * H::kPieces + 4 * kg;
 #pragma unroll
     for (int e = 0; e < 4; ++e) {
       uint4 o;
@@ -307,7 +334,7 @@ __device__ __forceinline__ void run_segment(const DecodeArgs& a, uint4* lds, int
     }
   } else {
     const int64_t row = slot * num_heads + head;
-    float4* prow = reinterpret_cast<float4*>(a.part_o + row * kHeadDim + 32 * kg);
+    float4* prow = reinterpret_cast<float4*>(a.part_o + row * D + 32 * kg);
 #pragma unroll
     for (int e = 0; e < 4; ++e) {
       prow[2 * e] = make_float4(acc[0][e], acc[1][e], acc[2][e], acc[3][e]);
@@ -320,10 +347,10 @@ __device__ __forceinline__ void run_segment(const DecodeArgs& a, uint4* lds, int
 // Fixed-chunk split: grid.x = batch * max_chunks, grid.y = num_kv_heads / NW,
 // block = NW * 64.  Workgroup (b, c) owns positions [c*chunk, (c+1)*chunk) of
 // sequence b; partial slot = b * max_chunks + c.
-template <int NW>
+template <int NW, int D>
 __global__ __launch_bounds__(NW * 64) void paged_decode_splitk_kernel(DecodeArgs a, int chunk,
                                                                       int max_chunks) {
-  __shared__ uint4 k_tile[NW][kStep * kLdsRowPieces];
+  __shared__ uint4 k_tile[NW][kStep * HeadDim<D>::kLdsRowPieces];
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int lane = threadIdx.x & 63;
   const int b = blockIdx.x / max_chunks;
@@ -334,8 +361,8 @@ __global__ __launch_bounds__(NW * 64) void paged_decode_splitk_kernel(DecodeArgs
   if (t0 >= ctx) return;  // also every chunk of an empty sequence
   const int t1 = min(ctx, t0 + chunk);
   const bool direct = ctx <= chunk;
-  run_segment(a, k_tile[wave], b, blockIdx.y * NW + wave, t0, t1,
-              (int64_t)b * max_chunks + c, direct, lane & 15, lane >> 4);
+  run_segment<D>(a, k_tile[wave], b, blockIdx.y * NW + wave, t0, t1,
+                 (int64_t)b * max_chunks + c, direct, lane);
 }
 
 // Inclusive prefix sum over the 64 lanes of a wave with DPP moves: a
@@ -363,12 +390,12 @@ __device__ __forceinline__ int wave_inclusive_scan(int x) {
 // never needs the lengths.  Workgroup 0 also leaves the exclusive prefix sums
 // (steps before each sequence, total at [batch]) in `prefix` for the combine
 // pass.  grid.x = num_wgs, grid.y = num_kv_heads / NW, block = NW * 64.
-template <int NW>
+template <int NW, int D>
 __global__ __launch_bounds__(NW * 64) void paged_decode_balanced_kernel(DecodeArgs a, int batch,
                                                                         int num_wgs,
                                                                         int min_steps,
                                                                         int32_t* prefix) {
-  __shared__ uint4 k_tile[NW][kStep * kLdsRowPieces];
+  __shared__ uint4 k_tile[NW][kStep * HeadDim<D>::kLdsRowPieces];
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int lane = threadIdx.x & 63;
   const int g = blockIdx.x;
@@ -468,8 +495,8 @@ __global__ __launch_bounds__(NW * 64) void paged_decode_balanced_kernel(DecodeAr
     const int t0 = __builtin_amdgcn_readfirstlane((pos - before) * kStep);
     const int t1 = __builtin_amdgcn_readfirstlane(min(ctx, (seg_end - before) * kStep));
     const bool direct = pos == before && seg_end == before + nb;
-    run_segment(a, k_tile[wave], sb, blockIdx.y * NW + wave, t0, t1, (int64_t)(g + sb), direct,
-                lane & 15, lane >> 4);
+    run_segment<D>(a, k_tile[wave], sb, blockIdx.y * NW + wave, t0, t1, (int64_t)(g + sb),
+                   direct, lane);
     pos = seg_end;
   }
 }
@@ -480,12 +507,13 @@ __global__ __launch_bounds__(NW * 64) void paged_decode_balanced_kernel(DecodeAr
 // mode: they are slots g_first + b .. g_last + b, where g_first..g_last are the
 // workgroups whose runs of `run` steps touch the sequence.  A sequence with one
 // partial was written by the split kernel itself; an empty one gives zeros.
-__global__ __launch_bounds__(kHeadDim) void paged_decode_combine_kernel(
+__global__ __launch_bounds__(kMaxHeadDim) void paged_decode_combine_kernel(
     const float* __restrict__ part_o, const float* __restrict__ part_ml,
     const int32_t* __restrict__ context_lens, const int32_t* __restrict__ prefix,
     uint16_t* __restrict__ out, int num_heads, int chunk, int max_chunks, int max_positions,
     int batch, int num_wgs, int min_steps, float scale_log2e) {
   const int b = blockIdx.x, h = blockIdx.y, d = threadIdx.x;
+  const int head_dim = blockDim.x;
   int nparts;
   int64_t first;
   if (prefix == nullptr) {
@@ -500,7 +528,7 @@ __global__ __launch_bounds__(kHeadDim) void paged_decode_combine_kernel(
     first = (int64_t)g_first + b;
   }
   if (nparts == 1) return;  // written by the split kernel itself
-  uint16_t* o = out + ((int64_t)b * num_heads + h) * kHeadDim + d;
+  uint16_t* o = out + ((int64_t)b * num_heads + h) * head_dim + d;
   if (nparts == 0) {  // empty sequence: 0 / (0 + 1e-9)
     *o = 0;
     return;
@@ -517,7 +545,7 @@ __global__ __launch_bounds__(kHeadDim) void paged_decode_combine_kernel(
     for (int i = 0; i < 8; ++i) {
       const int64_t row = base + (int64_t)min(c0 + i, nparts - 1) * num_heads;
       mlv[i] = ml[row];
-      po[i] = part_o[row * kHeadDim + d];
+      po[i] = part_o[row * head_dim + d];
     }
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
@@ -558,13 +586,13 @@ struct WorkspacePlan {
   size_t bytes;
 };
 
-bool plan_workspace(int64_t batch, int64_t num_heads, int64_t max_blocks, int64_t block_size,
-                    int chunk, WorkspacePlan* plan) {
+bool plan_workspace(int64_t batch, int64_t num_heads, int64_t head_dim, int64_t max_blocks,
+                    int64_t block_size, int chunk, WorkspacePlan* plan) {
   if (chunk == 0) {
     plan->num_wgs = balanced_workgroups(batch, max_blocks, block_size);
     plan->max_chunks = 0;
     plan->slots = plan->num_wgs + batch;
-    const size_t floats = (size_t)plan->slots * num_heads * (kHeadDim + 2);
+    const size_t floats = (size_t)plan->slots * num_heads * (head_dim + 2);
     plan->bytes = floats * sizeof(float) + (size_t)(batch + 1) * sizeof(int32_t);
     return batch * ((max_blocks * block_size + kStep - 1) / kStep) <= INT32_MAX;
   }
@@ -573,7 +601,7 @@ bool plan_workspace(int64_t batch, int64_t num_heads, int64_t max_blocks, int64_
   plan->num_wgs = 0;
   plan->max_chunks = (int)mc;
   plan->slots = batch * mc;
-  plan->bytes = (size_t)plan->slots * num_heads * (kHeadDim + 2) * sizeof(float);
+  plan->bytes = (size_t)plan->slots * num_heads * (head_dim + 2) * sizeof(float);
   return true;
 }
 
@@ -597,11 +625,11 @@ extern "C" size_t nvj_paged_decode_workspace_bytes(int32_t batch, int32_t num_he
                                                    int32_t head_dim, int32_t max_blocks,
                                                    int32_t block_size, int32_t num_kv_heads,
                                                    int32_t chunk) {
-  if (batch <= 0 || num_heads <= 0 || head_dim != kHeadDim || max_blocks <= 0 ||
+  if (batch <= 0 || num_heads <= 0 || (head_dim != 128 && head_dim != 64) || max_blocks <= 0 ||
       block_size <= 0 || num_kv_heads <= 0 || chunk < 0 || chunk % kStep != 0)
     return 0;
   WorkspacePlan plan;
-  if (!plan_workspace(batch, num_heads, max_blocks, block_size, chunk, &plan)) return 0;
+  if (!plan_workspace(batch, num_heads, head_dim, max_blocks, block_size, chunk, &plan)) return 0;
   return plan.bytes;
 }
 
@@ -619,7 +647,8 @@ extern "C" int nvj_paged_decode_launch_phases(void* stream, const void* q, const
     return NVJ_ERR_BAD_SHAPE;
   if (num_heads % num_kv_heads != 0) return NVJ_ERR_BAD_SHAPE;
   const int group = num_heads / num_kv_heads;
-  if (head_dim != kHeadDim || group > 16 || block_size % kStep != 0 || chunk % kStep != 0)
+  if ((head_dim != 128 && head_dim != 64) || group > 16 || block_size % kStep != 0 ||
+      chunk % kStep != 0)
     return NVJ_ERR_UNSUPPORTED;
   if ((int64_t)max_blocks * block_size > INT32_MAX) return NVJ_ERR_BAD_SHAPE;
   if (batch == 0) return NVJ_OK;
@@ -651,48 +680,52 @@ extern "C" int nvj_paged_decode_launch_phases(void* stream, const void* q, const
   WorkspacePlan plan = {0, 1, 0, 0};
   int32_t* prefix = nullptr;
   if (max_blocks > 0) {
-    if (!plan_workspace(batch, num_heads, max_blocks, block_size, chunk, &plan))
+    if (!plan_workspace(batch, num_heads, head_dim, max_blocks, block_size, chunk, &plan))
       return NVJ_ERR_BAD_SHAPE;
     if (!workspace || workspace_bytes < plan.bytes) return NVJ_ERR_WORKSPACE;
     a.part_o = static_cast<float*>(workspace);
-    a.part_ml = a.part_o + plan.slots * num_heads * kHeadDim;
+    a.part_ml = a.part_o + plan.slots * num_heads * head_dim;
     if (chunk == 0) prefix = reinterpret_cast<int32_t*>(a.part_ml + plan.slots * num_heads * 2);
 
     if (phases & NVJ_PHASE_SPLITK) {
       const int nw =
           num_kv_heads % 8 == 0 ? 8 : num_kv_heads % 4 == 0 ? 4 : num_kv_heads % 2 == 0 ? 2 : 1;
       const unsigned gy = (unsigned)(num_kv_heads / nw);
+      // one instantiation per (waves per workgroup, head_dim)
+#define NVJ_FOR_SHAPE(LAUNCH)                 \
+  switch (nw * 1000 + head_dim) {             \
+    case 8128: LAUNCH(8, 128); break;         \
+    case 4128: LAUNCH(4, 128); break;         \
+    case 2128: LAUNCH(2, 128); break;         \
+    case 1128: LAUNCH(1, 128); break;         \
+    case 8064: LAUNCH(8, 64); break;          \
+    case 4064: LAUNCH(4, 64); break;          \
+    case 2064: LAUNCH(2, 64); break;          \
+    default: LAUNCH(1, 64); break;            \
+  }
       if (chunk == 0) {
         const dim3 grid((unsigned)plan.num_wgs, gy);
-#define NVJ_LAUNCH(NWV)                                               \
-  paged_decode_balanced_kernel<NWV><<<grid, dim3(NWV * 64), 0, s>>>( \
+#define NVJ_LAUNCH_BALANCED(NWV, DV)                                      \
+  paged_decode_balanced_kernel<NWV, DV><<<grid, dim3(NWV * 64), 0, s>>>( \
       a, batch, plan.num_wgs, kMinBalancedSteps, prefix)
-        switch (nw) {
-          case 8: NVJ_LAUNCH(8); break;
-          case 4: NVJ_LAUNCH(4); break;
-          case 2: NVJ_LAUNCH(2); break;
-          default: NVJ_LAUNCH(1); break;
-        }
-#undef NVJ_LAUNCH
+        NVJ_FOR_SHAPE(NVJ_LAUNCH_BALANCED)
+#undef NVJ_LAUNCH_BALANCED
       } else {
         const dim3 grid((unsigned)(batch * plan.max_chunks), gy);
-#define NVJ_LAUNCH(NWV) \
-  paged_decode_splitk_kernel<NWV><<<grid, dim3(NWV * 64), 0, s>>>(a, chunk, plan.max_chunks)
-        switch (nw) {
-          case 8: NVJ_LAUNCH(8); break;
-          case 4: NVJ_LAUNCH(4); break;
-          case 2: NVJ_LAUNCH(2); break;
-          default: NVJ_LAUNCH(1); break;
-        }
-#undef NVJ_LAUNCH
+#define NVJ_LAUNCH_FIXED(NWV, DV)                                                    \
+  paged_decode_splitk_kernel<NWV, DV><<<grid, dim3(NWV * 64), 0, s>>>(a, chunk, \
+                                                                       plan.max_chunks)
+        NVJ_FOR_SHAPE(NVJ_LAUNCH_FIXED)
+#undef NVJ_LAUNCH_FIXED
       }
+#undef NVJ_FOR_SHAPE
       if (hipGetLastError() != hipSuccess) return NVJ_ERR_LAUNCH;
     }
   } else {
     chunk = kStep;  // no pages at all: every sequence is empty, combine writes zeros
   }
   if (!(phases & NVJ_PHASE_COMBINE)) return NVJ_OK;
-  paged_decode_combine_kernel<<<dim3((unsigned)batch, (unsigned)num_heads), dim3(kHeadDim), 0, s>>>(
+  paged_decode_combine_kernel<<<dim3((unsigned)batch, (unsigned)num_heads), dim3(head_dim), 0, s>>>(
       a.part_o, a.part_ml, context_lens, prefix, static_cast<uint16_t*>(out), num_heads, chunk,
       plan.max_chunks, max_blocks * block_size, batch, plan.num_wgs, kMinBalancedSteps,
       a.scale_log2e);

@@ -45,7 +45,7 @@ def test_argument_validation_without_a_gpu():
         return L(None, p, p, p, p, p, p, p, 1 << 30, a["batch"], a["Hq"], a["Hkv"], a["D"],
                  a["bs"], a["MB"], a["NB"], 0.1, kw.get("chunk", 0))
 
-    assert call(D=64) == -3                # head_dim not built
+    assert call(D=96) == -3                # head_dim not built (128 and 64 are)
     assert call(Hq=30) == -2               # Hq % Hkv
     assert call(Hq=256, Hkv=8) == -3       # group > 16
     assert call(bs=48) == -3

@@ -168,3 +168,55 @@ def test_balanced_split_all_empty_and_single_position():
     got = run_hip(q, kc, vc, bt, ctx2, 0.1, bs, 0)
     assert np.array_equal(got[4], np.repeat(vc[bt[4, 0], 0], Hq // Hkv, axis=0))
     assert not np.delete(got, 4, axis=0).any()
+
+
+def test_reference_parity_check_shape_d64():
+    """Shape of the reference's only numeric parity check
+    (layers/pallas_attention.py:622-647): B=4, Hq=8, Hkv=2, D=64, 32 pages of 256,
+    4 pages per sequence in order, ctx = [200, 512, 300, 100], bf16."""
+    print("case reference parity shape D=64", flush=True)
+    from nanovllm_jax_amd.workloads import draw_bf16_bits
+    B, Hq, Hkv, D, bs, NB = 4, 8, 2, 64, 256, 32
+    rng = np.random.Generator(np.random.PCG64(42))
+    q = draw_bf16_bits(rng, (B, Hq, D))
+    kc = draw_bf16_bits(rng, (NB, bs, Hkv, D))
+    vc = draw_bf16_bits(rng, (NB, bs, Hkv, D))
+    bt = np.arange(16, dtype=np.int32).reshape(4, 4)
+    ctx = np.array([200, 512, 300, 100], np.int32)
+    scale = 1.0 / np.sqrt(D)
+    want = oracle(q, kc, vc, bt, ctx, scale, bs)
+    for chunk in (0, 64, 256):
+        got = run_hip(q, kc, vc, bt, ctx, scale, bs, chunk)
+        assert_close_bf16(got, want, what=f"D=64 chunk={chunk}")
+
+
+def test_reference_per_sequence_blocks_shape_d64_page64():
+    """Shape of the reference's TEST 4 (test_mosaic_kernels.py:234-260): B=4, Hq=8,
+    Hkv=2, D=64, 16 pages of 64, tables [[0..3],[4..7],[8..11],[12..15]],
+    ctx = [100, 150, 200, 250]."""
+    print("case reference per-sequence blocks shape D=64 page 64", flush=True)
+    from nanovllm_jax_amd.workloads import draw_bf16_bits
+    B, Hq, Hkv, D, bs, NB = 4, 8, 2, 64, 64, 16
+    rng = np.random.Generator(np.random.PCG64(43))
+    q = draw_bf16_bits(rng, (B, Hq, D))
+    kc = draw_bf16_bits(rng, (NB, bs, Hkv, D))
+    vc = draw_bf16_bits(rng, (NB, bs, Hkv, D))
+    bt = np.arange(16, dtype=np.int32).reshape(4, 4)
+    ctx = np.array([100, 150, 200, 250], np.int32)
+    scale = 1.0 / np.sqrt(D)
+    want = oracle(q, kc, vc, bt, ctx, scale, bs)
+    got = run_hip(q, kc, vc, bt, ctx, scale, bs, 0)
+    assert_close_bf16(got, want, what="D=64 page 64")
+
+
+@pytest.mark.parametrize("Hq,Hkv", [(8, 8), (16, 4), (8, 1)])
+def test_d64_random_groups_and_tails(Hq, Hkv):
+    print(f"case D=64 random Hq={Hq} Hkv={Hkv}", flush=True)
+    B, D, bs, NB = 5, 64, 32, 60
+    q, kc, vc, bt, ctx = make_problem(200 + Hq, B, Hq, Hkv, D, bs, NB, [1, 31, 33, 0, 700])
+    scale = 1.0 / np.sqrt(D)
+    want = oracle(q, kc, vc, bt, ctx, scale, bs)
+    for chunk in (0, 96):
+        got = run_hip(q, kc, vc, bt, ctx, scale, bs, chunk)
+        assert_close_bf16(got, want, what=f"D=64 Hq={Hq} Hkv={Hkv} chunk={chunk}")
+    assert np.array_equal(got[0], np.repeat(vc[bt[0, 0], 0], Hq // Hkv, axis=0))
