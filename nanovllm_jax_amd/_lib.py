@@ -44,6 +44,9 @@ SYMBOLS = {
     "nvj_advance_decode_launch": (_c.c_int, [
         _c.c_void_p, _c.c_void_p, _c.c_int32, _c.c_void_p, _c.c_void_p, _c.c_void_p, _c.c_void_p,
         _c.c_void_p, _c.c_int32, _c.c_int32, _c.c_int32]),
+    "nvj_prefill_attention_launch": (_c.c_int, [
+        _c.c_void_p, _c.c_void_p, _c.c_void_p, _c.c_void_p, _c.c_void_p, _c.c_void_p, _c.c_void_p,
+        _c.c_int32, _c.c_int32, _c.c_int32, _c.c_int32, _c.c_int32, _c.c_float]),
 }
 NVJ_PHASE_SPLITK = 1
 NVJ_PHASE_COMBINE = 2

@@ -1,0 +1,343 @@
+// Variable-length causal prefill attention for gfx950 (CDNA4, wave64).
+//
+// Stands in for variable_length_attention_prefill (layers/attention.py:135-279
+// of the reference) as called from Attention._prefill_attention (:331-364): q,
+// k, v are the packed rows of the prompts being prefilled, sequence i owning q
+// rows [cu_q[i], cu_q[i+1]) and k/v rows [cu_k[i], cu_k[i+1]).  Query position
+// p of a sequence attends key positions <= p of the same sequence (the
+// reference's mask `q_pos >= k_pos`, both counted from the start of the
+// sequence, :232-243).  GQA maps query head h to kv head h / G.  Nothing is
+// padded and nothing of size max_len^2 is materialised.
+//
+// MFMA-bound.  One workgroup = 4 waves = 128 query rows of one (sequence, query
+// head); a wave owns 32 rows as two groups of 16 MFMA columns.  Keys are walked
+// 32 at a time; the K tile and the V tile of a step are fetched once per
+// workgroup and staged in LDS (double-buffered, one barrier per step):
+//   * K as rows of 16-byte pieces (padded), read back as the A operand of
+//     S^T[key, q] = K . Q^T  (v_mfma_f32_16x16x32_bf16, Q^T of both groups in
+//     registers for the whole tile);
+//   * V already transposed into A operands of O^T[dim, q] += V^T . P^T: the
+//     loading lane holds 2 keys x 8 dims and writes, per dim, the 2-key pair
+//     where the operand of (dim group, key group) expects it.
+// Softmax is the fp32 online form on the accumulator layout; P^T comes out of
+// the S^T accumulators already in B-operand layout (same reduction-slot <-> key
+// map as the decode kernel).  Only tiles that touch the diagonal are masked.
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "nvj_paged_attn.h"
+
+namespace {
+
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
+typedef __attribute__((ext_vector_type(4))) float f32x4;
+
+constexpr int kD = 128;
+constexpr int kPieces = 16;          // 16-byte pieces per (position, head) row
+constexpr int kBM = 128;             // query rows per workgroup
+constexpr int kWaves = 4;
+constexpr int kRowsPerWave = kBM / kWaves;   // 32 = two column groups of 16
+constexpr int kKeys = 32;            // keys per step
+constexpr int kKRow = kPieces + 1;   // padded K row in LDS, in pieces
+constexpr float kNegBig = -1.0e30f;
+constexpr float kLog2e = 1.4426950408889634f;
+
+__device__ __forceinline__ bf16x8 as_bf16x8(uint4 v) { return __builtin_bit_cast(bf16x8, v); }
+
+__device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi) {
+  typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2;
+  bf16x2 p = {(__bf16)lo, (__bf16)hi};
+  return __builtin_bit_cast(uint32_t, p);
+}
+
+typedef const __attribute__((address_space(4))) int32_t* const_i32_ptr;
+
+// reduction slot j of key group kg stands for this key of the 32-key step
+__device__ __forceinline__ int slot_key(int kg, int j) {
+  return j < 4 ? 4 * kg + j : 16 + 4 * kg + (j - 4);
+}
+
+// Cooperative tile loads of a workgroup: K 2 pieces per thread, V 2 keys per
+// thread.  K item i of the 512 (key, piece) pairs of a step: key = i / 16,
+// piece = i % 16.  V: wave = key group, lane = (quarter qd = lane >> 4, piece
+// c = lane & 15): the two keys of reduction slots 2*qd and 2*qd + 1 of that key
+// group.  Keys are clamped to the last visible one, so nothing at or beyond
+// k_end is read.
+struct TileLoader {
+  const uint4* k_head;
+  const uint4* v_head;
+  int64_t row_pieces;
+  int last_key, tid, wave, r, qd;
+
+  __device__ __forceinline__ void issue(int step, uint4& k0, uint4& k1, uint4& v0,
+                                        uint4& v1) const {
+    const int ks = step * kKeys;
+    const int piece = tid % kPieces, key = tid / kPieces;   // items tid and tid + 256
+    k0 = k_head[(int64_t)min(ks + key, last_key) * row_pieces + piece];
+    k1 = k_head[(int64_t)min(ks + key + 16, last_key) * row_pieces + piece];
+    v0 = v_head[(int64_t)min(ks + slot_key(wave, 2 * qd), last_key) * row_pieces + r];
+    v1 = v_head[(int64_t)min(ks + slot_key(wave, 2 * qd + 1), last_key) * row_pieces + r];
+  }
+
+  __device__ __forceinline__ void stage(uint4* k_tile, uint4* vt_tile, const uint4& k0,
+                                        const uint4& k1, const uint4& v0,
+                                        const uint4& v1) const {
+    const int piece = tid % kPieces, key = tid / kPieces;
+    k_tile[key * kKRow + piece] = k0;
+    k_tile[(key + 16) * kKRow + piece] = k1;
+    // 2 keys x 8 dims -> per dim the (key0, key1) pair, at slot pair 2*qd of the
+    // operand of (dim jd, key group = wave, piece r)
+    uint32_t* vt32 = reinterpret_cast<uint32_t*>(vt_tile);
+    const int base = (wave * kPieces + r) * 4 + qd;
+    const int dim_stride = 4 * kPieces * 4;   // dwords between consecutive jd
+    vt32[base + 0 * dim_stride] = __builtin_amdgcn_perm(v1.x, v0.x, 0x05040100u);
+    vt32[base + 1 * dim_stride] = __builtin_amdgcn_perm(v1.x, v0.x, 0x07060302u);
+    vt32[base + 2 * dim_stride] = __builtin_amdgcn_perm(v1.y, v0.y, 0x05040100u);
+    vt32[base + 3 * dim_stride] = __builtin_amdgcn_perm(v1.y, v0.y, 0x07060302u);
+    vt32[base + 4 * dim_stride] = __builtin_amdgcn_perm(v1.z, v0.z, 0x05040100u);
+    vt32[base + 5 * dim_stride] = __builtin_amdgcn_perm(v1.z, v0.z, 0x07060302u);
+    vt32[base + 6 * dim_stride] = __builtin_amdgcn_perm(v1.w, v0.w, 0x05040100u);
+    vt32[base + 7 * dim_stride] = __builtin_amdgcn_perm(v1.w, v0.w, 0x07060302u);
+  }
+};
+
+struct PrefillArgs {
+  const uint4* q;       // [Tq, Hq, 16] pieces
+  const uint4* k;       // [Tk, Hkv, 16] pieces
+  const uint4* v;
+  uint4* out;           // [Tq, Hq, 16] pieces
+  const int32_t* cu_q;  // [B + 1]
+  const int32_t* cu_k;  // [B + 1]
+  int batch, num_heads, num_kv_heads, group;
+  float scale_log2e;
+};
+
+// grid.x = upper bound on the number of 128-row query tiles, grid.y = Hq.
+__global__ __launch_bounds__(kWaves * 64, 2) void prefill_attention_kernel(PrefillArgs a,
+                                                                        int num_tiles_bound) {
+  __shared__ uint4 k_lds[2][kKeys * kKRow];
+  __shared__ uint4 vt_lds[2][8 * 4 * kPieces];   // [dim-in-piece jd][key group][piece]
+
+  const int tid = threadIdx.x;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int lane = tid & 63;
+  const int r = lane & 15;
+  const int kg = lane >> 4;
+  const int head = blockIdx.y;
+  const int kvh = head / a.group;
+  const const_i32_ptr cu_q = (const_i32_ptr)(uintptr_t)a.cu_q;
+  const const_i32_ptr cu_k = (const_i32_ptr)(uintptr_t)a.cu_k;
+
+  // Later tiles of a sequence have more keys to walk: hand them out first.
+  const int tile_id = num_tiles_bound - 1 - (int)blockIdx.x;
+  int seq = -1, q0 = 0;
+  {
+    int before = 0;
+    for (int s = 0; s < a.batch; ++s) {
+      const int len = cu_q[s + 1] - cu_q[s];
+      const int nt = (max(len, 0) + kBM - 1) / kBM;
+      if (tile_id < before + nt) {
+        seq = s;
+        q0 = (tile_id - before) * kBM;
+        break;
+      }
+      before += nt;
+    }
+  }
+  if (seq < 0) return;   // beyond the real number of tiles
+  const int q_base = cu_q[seq], len_q = cu_q[seq + 1] - q_base;
+  const int k_base = cu_k[seq], len_k = max(cu_k[seq + 1] - k_base, 0);
+  const int q_end = min(q0 + kBM, len_q);           // rows [q0, q_end) are real
+  const int k_end = min(len_k, q_end);              // keys [0, k_end) are visible to some row
+  const int nsteps = (k_end + kKeys - 1) / kKeys;
+
+  // ---- Q^T of both column groups as B operands: column r of group g is row
+  // q0 + 32*wave + 16*g + r; rows beyond the sequence are zero ----
+  bf16x8 qreg[2][4];
+#pragma unroll
+  for (int g = 0; g < 2; ++g) {
+    const int row = q0 + kRowsPerWave * wave + 16 * g + r;
+    const uint4 zero = make_uint4(0u, 0u, 0u, 0u);
+    const uint4* qrow =
+        a.q + ((int64_t)(q_base + min(row, len_q - 1)) * a.num_heads + head) * kPieces;
+#pragma unroll
+    for (int s = 0; s < 4; ++s) {
+      const uint4 t = qrow[4 * s + kg];
+      qreg[g][s] = as_bf16x8(row < len_q ? t : zero);
+    }
+  }
+
+  const int64_t k_row_pieces = (int64_t)a.num_kv_heads * kPieces;
+  const uint4* k_head = a.k + ((int64_t)k_base * a.num_kv_heads + kvh) * kPieces;
+  const uint4* v_head = a.v + ((int64_t)k_base * a.num_kv_heads + kvh) * kPieces;
+
+  uint4 kld0, kld1, vld0, vld1;
+  const TileLoader ld = {k_head, v_head, k_row_pieces, k_end - 1, tid, wave, r, kg};
+
+  f32x4 acc[2][8];
+  float m_run[2], l_run[2];
+#pragma unroll
+  for (int g = 0; g < 2; ++g) {
+    m_run[g] = kNegBig;
+    l_run[g] = 0.f;
+#pragma unroll
+    for (int jd = 0; jd < 8; ++jd) acc[g][jd] = f32x4{0.f, 0.f, 0.f, 0.f};
+  }
+
+  if (nsteps > 0) {
+    ld.issue(0, kld0, kld1, vld0, vld1);
+    ld.stage(k_lds[0], vt_lds[0], kld0, kld1, vld0, vld1);
+    if (nsteps > 1) ld.issue(1, kld0, kld1, vld0, vld1);
+  }
+  __syncthreads();
+
+  const float sl2 = a.scale_log2e;
+  const int wave_row0 = q0 + kRowsPerWave * wave;   // first query row of this wave
+
+  for (int step = 0; step < nsteps; ++step) {
+    const int buf = step & 1;
+    const int ks = step * kKeys;
+    const uint4* kt = k_lds[buf];
+    const uint4* vt = vt_lds[buf];
+
+    // the wave has rows that see keys of this step only if its last row >= ks
+    if (wave_row0 + kRowsPerWave - 1 >= ks) {
+      bf16x8 ka[2][4];
+#pragma unroll
+      for (int s = 0; s < 4; ++s) {
+        ka[0][s] = as_bf16x8(kt[r * kKRow + 4 * s + kg]);
+        ka[1][s] = as_bf16x8(kt[(16 + r) * kKRow + 4 * s + kg]);
+      }
+      bf16x8 va[8];
+#pragma unroll
+      for (int jd = 0; jd < 8; ++jd) va[jd] = as_bf16x8(vt[(jd * 4 + kg) * kPieces + r]);
+
+      // masking is needed where the step reaches past a row of the wave
+      // (diagonal) or past the last key of the sequence
+      const bool need_mask = ks + kKeys - 1 > wave_row0 || ks + kKeys > k_end;
+#pragma unroll
+      for (int g = 0; g < 2; ++g) {
+        f32x4 s0 = {0.f, 0.f, 0.f, 0.f}, s1 = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int s = 0; s < 4; ++s) {
+          s0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ka[0][s], qreg[g][s], s0, 0, 0, 0);
+          s1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ka[1][s], qreg[g][s], s1, 0, 0, 0);
+        }
+        // lane = (query row, key group): keys ks + 4*kg + e and ks + 16 + 4*kg + e;
+        // `limit` = last key of this step the row may see
+        const int limit = min(wave_row0 + 16 * g + r, k_end - 1) - ks;
+        if (need_mask) {
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            if (4 * kg + e > limit) s0[e] = kNegBig;
+            if (16 + 4 * kg + e > limit) s1[e] = kNegBig;
+          }
+        }
+        float mx = fmaxf(fmaxf(fmaxf(s0[0], s0[1]), fmaxf(s0[2], s0[3])),
+                         fmaxf(fmaxf(s1[0], s1[1]), fmaxf(s1[2], s1[3])));
+        mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
+        mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+        const float m_new = fmaxf(m_run[g], mx);
+        const float alpha = __builtin_amdgcn_exp2f((m_run[g] - m_new) * sl2);
+        const float mneg = -m_new * sl2;
+        m_run[g] = m_new;
+        float p0[4], p1[4], psum = 0.f;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          p0[e] = __builtin_amdgcn_exp2f(fmaf(s0[e], sl2, mneg));
+          p1[e] = __builtin_amdgcn_exp2f(fmaf(s1[e], sl2, mneg));
+        }
+        if (need_mask) {
+          // masked entries weigh exactly 0 whatever the scale and even for a
+          // row whose running max is still the initial one
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            if (4 * kg + e > limit) p0[e] = 0.f;
+            if (16 + 4 * kg + e > limit) p1[e] = 0.f;
+          }
+        }
+#pragma unroll
+        for (int e = 0; e < 4; ++e) psum += p0[e] + p1[e];
+        l_run[g] = fmaf(l_run[g], alpha, psum);
+        uint4 pbits;
+        pbits.x = pack_bf16x2(p0[0], p0[1]);
+        pbits.y = pack_bf16x2(p0[2], p0[3]);
+        pbits.z = pack_bf16x2(p1[0], p1[1]);
+        pbits.w = pack_bf16x2(p1[2], p1[3]);
+        const bf16x8 pb = as_bf16x8(pbits);
+#pragma unroll
+        for (int jd = 0; jd < 8; ++jd) {
+          acc[g][jd] *= alpha;
+          acc[g][jd] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(va[jd], pb, acc[g][jd], 0, 0, 0);
+        }
+      }
+    }
+
+    // stage the next tile into the other buffer (last read one step ago, before
+    // the previous barrier), fetch the one after it, then meet the others
+    if (step + 1 < nsteps) {
+      ld.stage(k_lds[buf ^ 1], vt_lds[buf ^ 1], kld0, kld1, vld0, vld1);
+      if (step + 2 < nsteps) ld.issue(step + 2, kld0, kld1, vld0, vld1);
+    }
+    __syncthreads();
+  }
+
+  // ---- epilogue: acc[g][jd][e] is O[row][dim = 32*kg + 8*e + jd] ----
+#pragma unroll
+  for (int g = 0; g < 2; ++g) {
+    float l = l_run[g];
+    l += __shfl_xor(l, 16, 64);
+    l += __shfl_xor(l, 32, 64);
+    const int row = wave_row0 + 16 * g + r;
+    if (row < len_q) {
+      const float inv = l > 0.f ? 1.0f / l : 0.f;   // no visible key at all -> zeros
+      uint4* orow = a.out + ((int64_t)(q_base + row) * a.num_heads + head) * kPieces + 4 * kg;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        uint4 o;
+        o.x = pack_bf16x2(acc[g][0][e] * inv, acc[g][1][e] * inv);
+        o.y = pack_bf16x2(acc[g][2][e] * inv, acc[g][3][e] * inv);
+        o.z = pack_bf16x2(acc[g][4][e] * inv, acc[g][5][e] * inv);
+        o.w = pack_bf16x2(acc[g][6][e] * inv, acc[g][7][e] * inv);
+        orow[e] = o;
+      }
+    }
+  }
+}
+
+}  // namespace
+
+extern "C" int nvj_prefill_attention_launch(void* stream, const void* q, const void* k,
+                                            const void* v, const int32_t* cu_seqlens_q,
+                                            const int32_t* cu_seqlens_k, void* out,
+                                            int32_t total_q_tokens, int32_t batch,
+                                            int32_t num_heads, int32_t num_kv_heads,
+                                            int32_t head_dim, float scale) {
+  if (total_q_tokens < 0 || batch < 0 || num_heads <= 0 || num_kv_heads <= 0)
+    return NVJ_ERR_BAD_SHAPE;
+  if (num_heads % num_kv_heads != 0) return NVJ_ERR_BAD_SHAPE;
+  if (head_dim != kD) return NVJ_ERR_UNSUPPORTED;
+  if (total_q_tokens == 0 || batch == 0) return NVJ_OK;
+  if (!q || !k || !v || !cu_seqlens_q || !cu_seqlens_k || !out) return NVJ_ERR_NULL_POINTER;
+  if ((reinterpret_cast<uintptr_t>(q) | reinterpret_cast<uintptr_t>(k) |
+       reinterpret_cast<uintptr_t>(v) | reinterpret_cast<uintptr_t>(out)) & 15u)
+    return NVJ_ERR_BAD_SHAPE;
+  PrefillArgs a;
+  a.q = static_cast<const uint4*>(q);
+  a.k = static_cast<const uint4*>(k);
+  a.v = static_cast<const uint4*>(v);
+  a.out = static_cast<uint4*>(out);
+  a.cu_q = cu_seqlens_q;
+  a.cu_k = cu_seqlens_k;
+  a.batch = batch;
+  a.num_heads = num_heads;
+  a.num_kv_heads = num_kv_heads;
+  a.group = num_heads / num_kv_heads;
+  a.scale_log2e = scale * kLog2e;
+  // every sequence adds at most one partly filled tile
+  const int64_t tiles = (int64_t)total_q_tokens / kBM + batch;
+  if (tiles > INT32_MAX) return NVJ_ERR_BAD_SHAPE;
+  prefill_attention_kernel<<<dim3((unsigned)tiles, (unsigned)num_heads), dim3(kWaves * 64), 0,
+                             static_cast<hipStream_t>(stream)>>>(a, (int)tiles);
+  return hipGetLastError() == hipSuccess ? NVJ_OK : NVJ_ERR_LAUNCH;
+}

@@ -2,9 +2,9 @@
 
 Host-side mirror of ``layers/attention.py`` of the reference for the decode
 phase: ``store_kv_to_cache`` (:42-77) and ``Attention`` (:282-480) keep their
-names, argument order and return shapes.  Both run on the HIP library only;
-there is no prefill here (``context.is_prefill=True`` raises) and no alternate
-dispatch.
+names, argument order and return shapes, for the decode phase and for the
+prefill phase (:331-364).  Everything runs on the HIP library only; there is no
+alternate dispatch.
 
 Differences a caller can observe, both deliberate:
 * the cache is updated in place and the very same tensors are returned (the
@@ -19,6 +19,7 @@ import torch
 from .. import _lib
 from ..utils.context import AttentionContext
 from .paged_attention import paged_attention
+from .prefill_attention import variable_length_attention_prefill
 
 __all__ = ["store_kv_to_cache", "Attention"]
 
@@ -103,6 +104,15 @@ class Attention:
         self.k_cache = k_cache
         self.v_cache = v_cache
 
+    def _prefill_attention(self, q, k, v, context: AttentionContext):
+        """Variable-length causal attention over the packed prompt rows
+        (layers/attention.py:331-364)."""
+        dt = torch.bfloat16
+        return variable_length_attention_prefill(
+            q.to(dt).contiguous(), k.to(dt).contiguous(), v.to(dt).contiguous(),
+            context.cu_seqlens_q, context.cu_seqlens_k, context.max_seqlen_q,
+            context.max_seqlen_k, self.num_heads, self.num_kv_heads, self.scale)
+
     def _decode_attention(self, q, context: AttentionContext):
         q = q.to(self.k_cache.dtype)      # layers/attention.py:386-387
         return paged_attention(q, self.k_cache, self.v_cache, context.block_tables,
@@ -112,7 +122,7 @@ class Attention:
     def __call__(self, q, k, v, context: AttentionContext):
         if self.k_cache is None or self.v_cache is None:
             raise RuntimeError("set_kv_cache() must be called before the first decode step")
-        if context.is_prefill:
-            raise NotImplementedError("this package implements the decode phase only")
         store_kv_to_cache(k, v, self.k_cache, self.v_cache, context.slot_mapping)
+        if context.is_prefill:
+            return self._prefill_attention(q, k, v, context)
         return self._decode_attention(q, context)

@@ -1,0 +1,62 @@
+"""Variable-length causal prefill attention entry point.
+
+Host-side mirror of ``variable_length_attention_prefill``
+(``layers/attention.py:135-279`` of the reference): same argument list and
+result, one dispatch target: ``nvj_prefill_attention_launch``.  The static
+``max_seqlen_q / max_seqlen_k / batch_size`` arguments are accepted for
+signature compatibility; the HIP kernel pads nothing and does not need them.
+"""
+from __future__ import annotations
+
+import torch
+
+from .. import _lib
+
+__all__ = ["variable_length_attention_prefill"]
+
+
+def _require(cond: bool, msg: str) -> None:
+    if not cond:
+        raise ValueError(msg)
+
+
+def variable_length_attention_prefill(q, k, v, cu_seqlens_q, cu_seqlens_k, max_seqlen_q=0,
+                                      max_seqlen_k=0, num_heads=None, num_kv_heads=None,
+                                      scale=None, batch_size=None, *, out=None):
+    """q [total_tokens, num_heads, head_dim], k/v [total_k_tokens, num_kv_heads,
+    head_dim] bf16 packed rows; cu_seqlens_q / cu_seqlens_k [batch + 1] int32 on
+    the device.  Query position p of a sequence attends key positions <= p of the
+    same sequence.  Returns [total_tokens, num_heads, head_dim] bf16."""
+    lib = _lib.load()
+    for name, t, dt, nd in (("q", q, torch.bfloat16, 3), ("k", k, torch.bfloat16, 3),
+                            ("v", v, torch.bfloat16, 3),
+                            ("cu_seqlens_q", cu_seqlens_q, torch.int32, 1),
+                            ("cu_seqlens_k", cu_seqlens_k, torch.int32, 1)):
+        _require(isinstance(t, torch.Tensor), f"{name} must be a torch.Tensor")
+        _require(t.is_cuda, f"{name} must live on the GPU (got {t.device}); "
+                            "prefill attention has no CPU implementation")
+        _require(t.dtype == dt and t.dim() == nd and t.is_contiguous(),
+                 f"{name} must be contiguous {dt} with {nd} dims")
+        _require(t.device == q.device, f"{name} is on {t.device}, q on {q.device}")
+    total, hq, d = q.shape
+    _require(k.shape == v.shape and k.shape[2] == d, "k and v must share [tokens, kv_heads, head_dim]")
+    hkv = k.shape[1]
+    _require(num_heads in (None, hq) and num_kv_heads in (None, hkv), "head counts disagree with q/k")
+    _require(hq % hkv == 0, "num_heads must be a multiple of num_kv_heads")
+    batch = cu_seqlens_q.shape[0] - 1
+    _require(batch >= 0 and cu_seqlens_k.shape[0] == batch + 1, "cu_seqlens shapes disagree")
+    _require(batch_size in (None, batch), "batch_size disagrees with cu_seqlens")
+    if scale is None:
+        scale = d ** -0.5
+    if out is None:
+        out = torch.empty_like(q)
+    else:
+        _require(out.is_cuda and out.dtype == torch.bfloat16 and out.shape == q.shape
+                 and out.is_contiguous(), "out must match q")
+    with torch.cuda.device(q.device):
+        stream = torch.cuda.current_stream(q.device).cuda_stream
+        code = lib.nvj_prefill_attention_launch(
+            stream, q.data_ptr(), k.data_ptr(), v.data_ptr(), cu_seqlens_q.data_ptr(),
+            cu_seqlens_k.data_ptr(), out.data_ptr(), total, batch, hq, hkv, d, float(scale))
+    _lib.check(code, "nvj_prefill_attention_launch")
+    return out

@@ -11,7 +11,21 @@ from __future__ import annotations
 from dataclasses import dataclass
 from typing import Any
 
-__all__ = ["AttentionContext", "create_decode_context"]
+__all__ = ["AttentionContext", "create_decode_context", "create_prefill_context"]
+
+
+def _bucket_to_power_of_2(value: int, min_bucket: int = 16, max_bucket: int = 8192) -> int:
+    """Next power of two in [min_bucket, max_bucket] (``utils/context.py:18-32``:
+    the reference buckets its static max lengths to limit recompilation; kept so
+    that contexts carry the same values)."""
+    if value <= min_bucket:
+        return min_bucket
+    if value >= max_bucket:
+        return max_bucket
+    power = 1
+    while power < value:
+        power *= 2
+    return min(power, max_bucket)
 
 
 @dataclass
@@ -43,3 +57,14 @@ def create_decode_context(context_lens, slot_mapping, block_tables) -> Attention
     return AttentionContext(is_prefill=False, context_lens=context_lens,
                             slot_mapping=slot_mapping, block_tables=block_tables,
                             last_token_indices=None)
+
+
+def create_prefill_context(cu_seqlens_q, cu_seqlens_k, max_seqlen_q: int, max_seqlen_k: int,
+                           slot_mapping, block_tables=None) -> AttentionContext:
+    """Context for a prefill step (``utils/context.py:129-166``):
+    ``last_token_indices = cu_seqlens_q[1:] - 1``, max lengths bucketed."""
+    return AttentionContext(is_prefill=True, cu_seqlens_q=cu_seqlens_q, cu_seqlens_k=cu_seqlens_k,
+                            max_seqlen_q=_bucket_to_power_of_2(max_seqlen_q),
+                            max_seqlen_k=_bucket_to_power_of_2(max_seqlen_k),
+                            slot_mapping=slot_mapping, block_tables=block_tables,
+                            last_token_indices=cu_seqlens_q[1:] - 1)

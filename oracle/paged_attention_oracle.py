@@ -30,6 +30,13 @@ What pins each function (see tests/test_oracle_pinning.py):
                                   oracle's choice (the reference leaves it to
                                   XLA): PARITY UNPINNED at the level of fp32
                                   round-off of that sum.
+* ``variable_length_attention_prefill_ref``
+                                - fp64 brute force per (sequence, head, row);
+                                  torch ``scaled_dot_product_attention`` with
+                                  ``is_causal`` and ``enable_gqa``; row 0 is the
+                                  first V row; packing invariance (a batch equals
+                                  its sequences run one by one).  Same unpinned
+                                  bf16 rounding of probabilities as the fallback.
 * ``paged_attention_fallback_ref``
                                 - same checks; the bf16 rounding of the
                                   probabilities inside ``jax.nn.dot_product_attention``
@@ -56,6 +63,8 @@ __all__ = [
     "build_cos_sin_cache_ref",
     "qk_norm_rope_ref",
     "qk_norm_rope_store_ref",
+    "variable_length_attention_prefill_ref",
+    "textbook_prefill_f64",
     "prepare_decode_ref",
     "advance_decode_ref",
 ]
@@ -450,3 +459,74 @@ def advance_decode_ref(next_tokens, input_ids, positions, context_lens, slot_map
         ctx[i] = length
         slots[i] = page * block_size + (length - 1) % block_size
     return ids, pos, ctx, slots
+
+
+# ---------------------------------------------------------------------------
+# Variable-length causal prefill attention
+# ---------------------------------------------------------------------------
+
+def variable_length_attention_prefill_ref(q, k, v, cu_seqlens_q, cu_seqlens_k, scale,
+                                          return_f32: bool = False):
+    """Restates ``variable_length_attention_prefill`` (``layers/attention.py:135-279``)
+    without its padding: for sequence i, q rows [cu_q[i], cu_q[i+1]) attend k/v
+    rows [cu_k[i], cu_k[i+1]) under ``q_pos >= k_pos`` (:232-236, positions counted
+    from the start of the sequence) and the validity masks (:238-243).  Padding
+    rows exist only to make XLA shapes static (:186-222) and are scattered away
+    (:263-277), so leaving them out changes nothing.  The attention itself is
+    ``jax.nn.dot_product_attention`` (:247-251): fp32 logits from the bf16
+    operands, fp32 softmax, probabilities cast to bf16, fp32-accumulated PV,
+    bf16 result; GQA by head broadcast (h -> h // G).  A query row with no
+    visible key is not defined by the reference; zeros here.
+
+    q [T, Hq, D], k/v [Tk, Hkv, D] bf16 bits.  Returns [T, Hq, D] bf16 bits."""
+    q = np.asarray(q)
+    T, Hq, D = q.shape
+    Hkv = k.shape[1]
+    G = Hq // Hkv
+    cu_q = np.asarray(cu_seqlens_q, dtype=np.int64)
+    cu_k = np.asarray(cu_seqlens_k, dtype=np.int64)
+    out = np.zeros((T, Hq, D), dtype=np.float32)
+    scale = np.float32(scale)
+    for i in range(len(cu_q) - 1):
+        lq, lk = int(cu_q[i + 1] - cu_q[i]), int(cu_k[i + 1] - cu_k[i])
+        if lq <= 0 or lk <= 0:
+            continue
+        qs = bf16_bits_to_f32(q[cu_q[i]:cu_q[i + 1]]).reshape(lq, Hkv, G, D)
+        ks = bf16_bits_to_f32(k[cu_k[i]:cu_k[i + 1]])
+        vs = bf16_bits_to_f32(v[cu_k[i]:cu_k[i + 1]])
+        mask = np.arange(lq)[:, None] >= np.arange(lk)[None, :]           # :232-236
+        s = np.einsum("qhgd,khd->hgqk", qs, ks, dtype=np.float32) * scale
+        s = np.where(mask[None, None], s, np.float32(-1e30))
+        s = s - s.max(axis=-1, keepdims=True)
+        e = np.where(mask[None, None], np.exp(s, dtype=np.float32), np.float32(0))
+        p = e / e.sum(axis=-1, keepdims=True, dtype=np.float32)
+        p = bf16_bits_to_f32(f32_to_bf16_bits(p))                         # probs -> value dtype
+        o = np.einsum("hgqk,khd->qhgd", p, vs, dtype=np.float32)
+        out[cu_q[i]:cu_q[i + 1]] = o.reshape(lq, Hq, D)
+    return out if return_f32 else f32_to_bf16_bits(out)
+
+
+def textbook_prefill_f64(q, k, v, cu_seqlens_q, cu_seqlens_k, scale):
+    """Causal softmax(q K^T scale) V per (sequence, head, query row) in float64
+    with plain loops: the brute force the restatement above is pinned against."""
+    q = np.asarray(q)
+    T, Hq, D = q.shape
+    G = Hq // k.shape[1]
+    qf = bf16_bits_to_f32(q).astype(np.float64)
+    kf = bf16_bits_to_f32(np.asarray(k)).astype(np.float64)
+    vf = bf16_bits_to_f32(np.asarray(v)).astype(np.float64)
+    out = np.zeros((T, Hq, D))
+    for i in range(len(cu_seqlens_q) - 1):
+        q0, q1 = int(cu_seqlens_q[i]), int(cu_seqlens_q[i + 1])
+        k0, k1 = int(cu_seqlens_k[i]), int(cu_seqlens_k[i + 1])
+        for row in range(q1 - q0):
+            n = min(row + 1, k1 - k0)
+            if n <= 0:
+                continue
+            for h in range(Hq):
+                logits = np.array([float(scale) * (qf[q0 + row, h] @ kf[k0 + j, h // G])
+                                   for j in range(n)])
+                w = np.exp(logits - logits.max())
+                w /= w.sum()
+                out[q0 + row, h] = sum(w[j] * vf[k0 + j, h // G] for j in range(n))
+    return out

@@ -96,9 +96,8 @@ def test_host_mirror_refuses_cpu_tensors():
     with pytest.raises(RuntimeError, match="set_kv_cache"):
         attn(q, q, q, c)
     attn.set_kv_cache(kc, kc.clone())
-    c.is_prefill = True
-    with pytest.raises(NotImplementedError):
-        attn(q, q, q, c)
+    with pytest.raises(ValueError, match="GPU"):
+        attn(q, q[:, :8].contiguous(), q[:, :8].contiguous(), c)
 
 
 def test_missing_library_fails_loudly(monkeypatch, tmp_path):

@@ -335,3 +335,53 @@ def test_advance_decode_inactive_and_missing_page():
     i2, p2, c2, s2 = advance_decode_ref([70, 80, 90], ids, pos, ctx, slots, bt, bs)
     assert list(c2) == [4, 0, 5] and list(s2) == [-1, -1, 24]      # row 0: next page missing
     assert list(i2) == [7, 8, 90] and list(p2) == [3, 0, 4]
+
+
+# ---------------------------------------------------------------- prefill attention
+def _prefill_problem(seed, lens_q, lens_k, Hq, Hkv, D):
+    rng = np.random.Generator(np.random.PCG64(seed))
+    cu_q = np.concatenate([[0], np.cumsum(lens_q)]).astype(np.int32)
+    cu_k = np.concatenate([[0], np.cumsum(lens_k)]).astype(np.int32)
+    q = f32_to_bf16_bits(rng.standard_normal((cu_q[-1], Hq, D), dtype=np.float32))
+    k = f32_to_bf16_bits(rng.standard_normal((cu_k[-1], Hkv, D), dtype=np.float32))
+    v = f32_to_bf16_bits(rng.standard_normal((cu_k[-1], Hkv, D), dtype=np.float32))
+    return q, k, v, cu_q, cu_k
+
+
+@pytest.mark.parametrize("Hq,Hkv", [(2, 2), (4, 2), (4, 1)])
+def test_prefill_against_fp64_brute_force(Hq, Hkv):
+    from oracle.paged_attention_oracle import (textbook_prefill_f64,
+                                               variable_length_attention_prefill_ref)
+    lens = [1, 7, 12]
+    q, k, v, cu_q, cu_k = _prefill_problem(71 + Hq, lens, lens, Hq, Hkv, 16)
+    got = variable_length_attention_prefill_ref(q, k, v, cu_q, cu_k, 0.4, return_f32=True)
+    want = textbook_prefill_f64(q, k, v, cu_q, cu_k, 0.4)
+    np.testing.assert_allclose(got, want, atol=1e-2, rtol=1e-2)   # probabilities are rounded to bf16
+    # row 0 of every sequence sees one key: exactly its V row
+    for i in range(len(lens)):
+        np.testing.assert_allclose(got[cu_q[i]], np.repeat(bf16_bits_to_f32(v[cu_k[i]]), Hq // Hkv, 0),
+                                   rtol=1e-6, atol=0)
+    # unequal lengths: top-left aligned causal mask, keys beyond len_k never seen
+    q2, k2, v2, cq2, ck2 = _prefill_problem(75, [6, 3], [4, 9], Hq, Hkv, 16)
+    got2 = variable_length_attention_prefill_ref(q2, k2, v2, cq2, ck2, 0.4, return_f32=True)
+    np.testing.assert_allclose(got2, textbook_prefill_f64(q2, k2, v2, cq2, ck2, 0.4), atol=1e-2, rtol=1e-2)
+
+
+def test_prefill_against_torch_sdpa_causal_gqa_and_packing_invariance():
+    from oracle.paged_attention_oracle import variable_length_attention_prefill_ref
+    lens = [33, 5, 64]
+    Hq, Hkv, D = 8, 2, 32
+    q, k, v, cu_q, cu_k = _prefill_problem(81, lens, lens, Hq, Hkv, D)
+    got = variable_length_attention_prefill_ref(q, k, v, cu_q, cu_k, D ** -0.5, return_f32=True)
+    for i, n in enumerate(lens):
+        sl = slice(cu_q[i], cu_q[i + 1])
+        qq = bits_to_torch(q[sl]).float().permute(1, 0, 2)[None]
+        kk = bits_to_torch(k[sl]).float().permute(1, 0, 2)[None]
+        vv = bits_to_torch(v[sl]).float().permute(1, 0, 2)[None]
+        o = torch.nn.functional.scaled_dot_product_attention(qq, kk, vv, is_causal=True,
+                                                             enable_gqa=True)[0].permute(1, 0, 2)
+        np.testing.assert_allclose(got[sl], o.numpy(), atol=1e-2, rtol=1e-2)
+        # a batch is its sequences one by one
+        alone = variable_length_attention_prefill_ref(q[sl], k[sl], v[sl], [0, n], [0, n],
+                                                      D ** -0.5, return_f32=True)
+        assert np.array_equal(alone, got[sl])
