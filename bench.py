@@ -158,6 +158,48 @@ def bench_decode_step(args, torch):
     return 0
 
 
+MFMA_BF16_PEAK_TFLOPS = 2500.0
+
+
+def bench_prefill(args, torch):
+    """Variable-length causal prefill attention at the Qwen3-8B head shape
+    (Hq=32, Hkv=8, D=128): 8 prompts of 4096 tokens, packed.  Reports TFLOP/s
+    (4 * Hq * D flop per visible (query, key) pair) against the dense bf16 MFMA
+    peak."""
+    from nanovllm_jax_amd import variable_length_attention_prefill
+    dev = torch.device("cuda:0")
+    hq, hkv, d = 32, 8, 128
+    lens = [int(x) for x in args.prefill_lens.split(",")]
+    cu = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
+    g = torch.Generator(device=dev)
+    g.manual_seed(7)
+    total = int(cu[-1])
+    q = torch.randn((total, hq, d), generator=g, device=dev).to(torch.bfloat16)
+    k = torch.randn((total, hkv, d), generator=g, device=dev).to(torch.bfloat16)
+    v = torch.randn((total, hkv, d), generator=g, device=dev).to(torch.bfloat16)
+    cu_t = torch.from_numpy(cu).to(dev)
+    out = torch.empty_like(q)
+    fn = lambda: variable_length_attention_prefill(q, k, v, cu_t, cu_t, scale=d ** -0.5, out=out)
+    for _ in range(args.warmup):
+        fn()
+    ms, wall = timed(fn, args.steps, torch)
+    pairs = sum(n * (n + 1) // 2 for n in lens)
+    flops = 4.0 * hq * d * pairs
+    tflops = flops / (ms * 1e-3) / 1e12
+    rec = {"metric": "prefill attention TFLOP/s (causal, varlen, Qwen3-8B head shape)",
+           "value": round(tflops, 1), "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps,
+           "warmup": args.warmup, "ms_per_step": round(wall, 4), "higher_is_better": True,
+           "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
+           "config": {"workload": f"prefill: Hq={hq} Hkv={hkv} D={d}, prompt lengths {lens}",
+                      "flops_per_call": flops},
+           "roofline": {"bound": "mfma", "achieved": round(tflops, 1),
+                        "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
+                        "frac": round(tflops / MFMA_BF16_PEAK_TFLOPS, 4), "traffic": None,
+                        "kernel": "prefill_attention_kernel", "kernel_us": round(ms * 1e3, 1)}}
+    print(json.dumps(rec), flush=True)
+    return 0
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -171,6 +213,10 @@ def main():
                     help="also run a plain 1 GiB device-to-device copy a few times, so a "
                          "counter run has a kernel of known traffic to scale against")
     ap.add_argument("--cpu-budget", type=float, default=20.0)
+    ap.add_argument("--prefill", action="store_true",
+                    help="time the prefill attention kernel instead; prints its own JSON line")
+    ap.add_argument("--prefill-lens", default=",".join(["4096"] * 8),
+                    help="comma-separated prompt lengths for --prefill")
     ap.add_argument("--decode-step", action="store_true",
                     help="time the whole-model decode step (config C5) instead of the "
                          "attention call; prints its own JSON line")
@@ -194,6 +240,8 @@ def main():
     torch.cuda.set_device(dev)
     if args.decode_step:
         return bench_decode_step(args, torch)
+    if args.prefill:
+        return bench_prefill(args, torch)
     w = make_workload(args.workload)
     q, kc, vc, bt, ctx, slots, k_new, v_new = device_inputs(w, torch, dev)
     chunk = args.chunk
