@@ -244,7 +244,7 @@ NVJ_API int nvj_advance_decode_launch(void* stream, const void* next_tokens,
  * key (its sequence has no k rows) gives zeros.  The static max_seqlen_q /
  * max_seqlen_k of the reference are not needed: nothing is padded.
  * total_q_tokens bounds the launch and must be >= cu_seqlens_q[batch].
- * head_dim must be 128.
+ * head_dim must be 128, scale >= 0.
  */
 NVJ_API int nvj_prefill_attention_launch(void* stream, const void* q, const void* k,
                             const void* v, const int32_t* cu_seqlens_q,

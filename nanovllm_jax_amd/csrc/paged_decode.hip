@@ -651,6 +651,7 @@ extern "C" int nvj_paged_decode_launch_phases(void* stream, const void* q, const
       chunk % kStep != 0)
     return NVJ_ERR_UNSUPPORTED;
   if ((int64_t)max_blocks * block_size > INT32_MAX) return NVJ_ERR_BAD_SHAPE;
+  if (!(scale >= 0.f)) return NVJ_ERR_BAD_SHAPE;   // the running max assumes a non-negative scale
   if (batch == 0) return NVJ_OK;
   if (!q || !k_cache || !v_cache || !context_lens || !out) return NVJ_ERR_NULL_POINTER;
   if (max_blocks > 0 && !block_tables) return NVJ_ERR_NULL_POINTER;

@@ -40,6 +40,7 @@ constexpr int kRowsPerWave = kBM / kWaves;   // 32 = two column groups of 16
 constexpr int kKeys = 32;            // keys per step
 constexpr int kKRow = kPieces + 1;   // padded K row in LDS, in pieces
 constexpr float kNegBig = -1.0e30f;
+constexpr float kLazyLog2 = 8.0f;    // running max moves only for gains above 2^8
 constexpr float kLog2e = 1.4426950408889634f;
 
 __device__ __forceinline__ bf16x8 as_bf16x8(uint4 v) { return __builtin_bit_cast(bf16x8, v); }
@@ -64,19 +65,36 @@ __device__ __forceinline__ int slot_key(int kg, int j) {
 // group.  Keys are clamped to the last visible one, so nothing at or beyond
 // k_end is read.
 struct TileLoader {
-  const uint4* k_head;
-  const uint4* v_head;
-  int64_t row_pieces;
+  const char* k_head;   // first key row of the sequence for this kv head
+  const char* v_head;
+  uint32_t row_bytes;   // bytes between consecutive keys
   int last_key, tid, wave, r, qd;
 
+  // Full tiles: uniform 64-bit base (ks rows) + one 32-bit lane offset per
+  // load; the last tile clamps every key to last_key.
   __device__ __forceinline__ void issue(int step, uint4& k0, uint4& k1, uint4& v0,
                                         uint4& v1) const {
     const int ks = step * kKeys;
-    const int piece = tid % kPieces, key = tid / kPieces;   // items tid and tid + 256
-    k0 = k_head[(int64_t)min(ks + key, last_key) * row_pieces + piece];
-    k1 = k_head[(int64_t)min(ks + key + 16, last_key) * row_pieces + piece];
-    v0 = v_head[(int64_t)min(ks + slot_key(wave, 2 * qd), last_key) * row_pieces + r];
-    v1 = v_head[(int64_t)min(ks + slot_key(wave, 2 * qd + 1), last_key) * row_pieces + r];
+    const uint32_t piece_bytes = (uint32_t)(tid % kPieces) * 16u;
+    const int key = tid / kPieces;   // items tid and tid + 256
+    const int vk0 = slot_key(wave, 2 * qd), vk1 = slot_key(wave, 2 * qd + 1);
+    if (ks + kKeys - 1 <= last_key) {
+      const char* kb = k_head + (size_t)ks * row_bytes;
+      const char* vb = v_head + (size_t)ks * row_bytes;
+      k0 = *reinterpret_cast<const uint4*>(kb + ((uint32_t)key * row_bytes + piece_bytes));
+      k1 = *reinterpret_cast<const uint4*>(kb + ((uint32_t)(key + 16) * row_bytes + piece_bytes));
+      v0 = *reinterpret_cast<const uint4*>(vb + ((uint32_t)vk0 * row_bytes + (uint32_t)r * 16u));
+      v1 = *reinterpret_cast<const uint4*>(vb + ((uint32_t)vk1 * row_bytes + (uint32_t)r * 16u));
+    } else {
+      k0 = *reinterpret_cast<const uint4*>(
+          k_head + (size_t)min(ks + key, last_key) * row_bytes + piece_bytes);
+      k1 = *reinterpret_cast<const uint4*>(
+          k_head + (size_t)min(ks + key + 16, last_key) * row_bytes + piece_bytes);
+      v0 = *reinterpret_cast<const uint4*>(
+          v_head + (size_t)min(ks + vk0, last_key) * row_bytes + (uint32_t)r * 16u);
+      v1 = *reinterpret_cast<const uint4*>(
+          v_head + (size_t)min(ks + vk1, last_key) * row_bytes + (uint32_t)r * 16u);
+    }
   }
 
   __device__ __forceinline__ void stage(uint4* k_tile, uint4* vt_tile, const uint4& k0,
@@ -167,12 +185,14 @@ __global__ __launch_bounds__(kWaves * 64, 2) void prefill_attention_kernel(Prefi
     }
   }
 
-  const int64_t k_row_pieces = (int64_t)a.num_kv_heads * kPieces;
-  const uint4* k_head = a.k + ((int64_t)k_base * a.num_kv_heads + kvh) * kPieces;
-  const uint4* v_head = a.v + ((int64_t)k_base * a.num_kv_heads + kvh) * kPieces;
+  const uint32_t row_bytes = (uint32_t)a.num_kv_heads * (kD * 2);
+  const char* k_head =
+      reinterpret_cast<const char*>(a.k + ((int64_t)k_base * a.num_kv_heads + kvh) * kPieces);
+  const char* v_head =
+      reinterpret_cast<const char*>(a.v + ((int64_t)k_base * a.num_kv_heads + kvh) * kPieces);
 
   uint4 kld0, kld1, vld0, vld1;
-  const TileLoader ld = {k_head, v_head, k_row_pieces, k_end - 1, tid, wave, r, kg};
+  const TileLoader ld = {k_head, v_head, row_bytes, k_end - 1, tid, wave, r, kg};
 
   f32x4 acc[2][8];
   float m_run[2], l_run[2];
@@ -237,10 +257,22 @@ __global__ __launch_bounds__(kWaves * 64, 2) void prefill_attention_kernel(Prefi
                          fmaxf(fmaxf(s1[0], s1[1]), fmaxf(s1[2], s1[3])));
         mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
         mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
-        const float m_new = fmaxf(m_run[g], mx);
-        const float alpha = __builtin_amdgcn_exp2f((m_run[g] - m_new) * sl2);
-        const float mneg = -m_new * sl2;
-        m_run[g] = m_new;
+        // Lazy running max: the reference point of the exponentials only moves
+        // when some row's block max exceeds it by more than 2^kLazyLog2 (a
+        // wave-uniform decision), so most steps skip the rescale of O^T and l.
+        // Probabilities may then exceed 1 (by at most that factor); the final
+        // O / l is unchanged because both carry the same reference.
+        const bool move = __any((mx - m_run[g]) * sl2 > kLazyLog2);
+        float mneg = -m_run[g] * sl2;
+        if (move) {
+          const float m_new = fmaxf(m_run[g], mx);
+          const float alpha = __builtin_amdgcn_exp2f((m_run[g] - m_new) * sl2);
+          m_run[g] = m_new;
+          mneg = -m_new * sl2;
+          l_run[g] *= alpha;
+#pragma unroll
+          for (int jd = 0; jd < 8; ++jd) acc[g][jd] *= alpha;
+        }
         float p0[4], p1[4], psum = 0.f;
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
@@ -258,7 +290,7 @@ __global__ __launch_bounds__(kWaves * 64, 2) void prefill_attention_kernel(Prefi
         }
 #pragma unroll
         for (int e = 0; e < 4; ++e) psum += p0[e] + p1[e];
-        l_run[g] = fmaf(l_run[g], alpha, psum);
+        l_run[g] += psum;
         uint4 pbits;
         pbits.x = pack_bf16x2(p0[0], p0[1]);
         pbits.y = pack_bf16x2(p0[2], p0[3]);
@@ -266,10 +298,8 @@ __global__ __launch_bounds__(kWaves * 64, 2) void prefill_attention_kernel(Prefi
         pbits.w = pack_bf16x2(p1[2], p1[3]);
         const bf16x8 pb = as_bf16x8(pbits);
 #pragma unroll
-        for (int jd = 0; jd < 8; ++jd) {
-          acc[g][jd] *= alpha;
+        for (int jd = 0; jd < 8; ++jd)
           acc[g][jd] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(va[jd], pb, acc[g][jd], 0, 0, 0);
-        }
       }
     }
 
@@ -317,6 +347,7 @@ extern "C" int nvj_prefill_attention_launch(void* stream, const void* q, const v
     return NVJ_ERR_BAD_SHAPE;
   if (num_heads % num_kv_heads != 0) return NVJ_ERR_BAD_SHAPE;
   if (head_dim != kD) return NVJ_ERR_UNSUPPORTED;
+  if (!(scale >= 0.f)) return NVJ_ERR_BAD_SHAPE;   // the running max assumes a non-negative scale
   if (total_q_tokens == 0 || batch == 0) return NVJ_OK;
   if (!q || !k || !v || !cu_seqlens_q || !cu_seqlens_k || !out) return NVJ_ERR_NULL_POINTER;
   if ((reinterpret_cast<uintptr_t>(q) | reinterpret_cast<uintptr_t>(k) |
