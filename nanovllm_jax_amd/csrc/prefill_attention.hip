@@ -130,7 +130,7 @@ struct PrefillArgs {
   float scale_log2e;
 };
 
-// grid.x = upper bound on the number of 128-row query tiles, grid.y = Hq.
+// grid.x = 8 * ceil(tile bound * Hq / 8) workgroups (see the work-item mapping below).
 __global__ __launch_bounds__(kWaves * 64, 2) void prefill_attention_kernel(PrefillArgs a,
                                                                         int num_tiles_bound) {
   __shared__ uint4 k_lds[2][kKeys * kKRow];
@@ -141,13 +141,26 @@ __global__ __launch_bounds__(kWaves * 64, 2) void prefill_attention_kernel(Prefi
   const int lane = tid & 63;
   const int r = lane & 15;
   const int kg = lane >> 4;
-  const int head = blockIdx.y;
-  const int kvh = head / a.group;
   const const_i32_ptr cu_q = (const_i32_ptr)(uintptr_t)a.cu_q;
   const const_i32_ptr cu_k = (const_i32_ptr)(uintptr_t)a.cu_k;
 
-  // Later tiles of a sequence have more keys to walk: hand them out first.
-  const int tile_id = num_tiles_bound - 1 - (int)blockIdx.x;
+  // Work item -> workgroup, XCD-aware.  Consecutive workgroup ids land on
+  // different XCDs (8 of them, each with its own L2), so the work list is cut
+  // into 8 contiguous parts and workgroup id L takes item (L % 8) * part + L / 8:
+  // one XCD then walks neighbouring items.  Items are ordered (kv head, query
+  // tile, query head of the group): neighbours share the K/V rows of one
+  // (sequence, kv head), which stay in that XCD's L2 instead of being fetched
+  // by all eight.  Later tiles of a sequence have more keys to walk and come
+  // first.
+  const int total_items = num_tiles_bound * a.num_heads;
+  const int part = (total_items + 7) / 8;
+  const int item = ((int)blockIdx.x % 8) * part + (int)blockIdx.x / 8;
+  if (item >= total_items) return;
+  const int per_kv_head = num_tiles_bound * a.group;
+  const int kvh = item / per_kv_head;
+  const int in_kv = item - kvh * per_kv_head;
+  const int tile_id = num_tiles_bound - 1 - in_kv / a.group;
+  const int head = kvh * a.group + in_kv % a.group;
   int seq = -1, q0 = 0;
   {
     int before = 0;
@@ -368,7 +381,10 @@ extern "C" int nvj_prefill_attention_launch(void* stream, const void* q, const v
   // every sequence adds at most one partly filled tile
   const int64_t tiles = (int64_t)total_q_tokens / kBM + batch;
   if (tiles > INT32_MAX) return NVJ_ERR_BAD_SHAPE;
-  prefill_attention_kernel<<<dim3((unsigned)tiles, (unsigned)num_heads), dim3(kWaves * 64), 0,
+  const int64_t items = tiles * num_heads;
+  if (items > INT32_MAX - 8) return NVJ_ERR_BAD_SHAPE;
+  const unsigned grid = (unsigned)((items + 7) / 8 * 8);
+  prefill_attention_kernel<<<dim3(grid), dim3(kWaves * 64), 0,
                              static_cast<hipStream_t>(stream)>>>(a, (int)tiles);
   return hipGetLastError() == hipSuccess ? NVJ_OK : NVJ_ERR_LAUNCH;
 }
