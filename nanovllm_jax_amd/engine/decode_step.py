@@ -27,11 +27,12 @@ import torch.nn.functional as F
 from .. import _lib
 from ..layers.attention import Attention
 from ..layers.paged_attention import paged_attention, paged_decode_workspace_bytes
+from ..layers.prefill_attention import variable_length_attention_prefill
 from ..layers.qk_rope_store import qk_norm_rope_store
-from ..utils.context import AttentionContext, create_decode_context
+from ..utils.context import AttentionContext, create_decode_context, create_prefill_context
 
 __all__ = ["DecodeModelConfig", "DecodeStepRunner", "prepare_block_tables", "prepare_decode",
-           "advance_decode"]
+           "prepare_prefill", "advance_decode"]
 
 
 @dataclass
@@ -75,6 +76,28 @@ def prepare_decode(last_tokens, seq_lens, block_tables, block_size):
         last_block_tokens = length - (len(table) - 1) * block_size
         slot_mapping[i] = table[-1] * block_size + last_block_tokens - 1
     return input_ids, positions, context_lens, slot_mapping, prepare_block_tables(block_tables)
+
+
+def prepare_prefill(token_lists, block_tables, block_size):
+    """Host filler of one prefill step without prefix caching
+    (``engine/model_runner.py:248-332`` with ``num_cached_tokens == 0``): packed
+    ``input_ids`` and ``positions = 0 .. len-1``, ``cu_seqlens_q == cu_seqlens_k``,
+    and per sequence the slots of its pages in order, ``block_size`` per page
+    except ``last_block_num_tokens`` in the last (:300-309)."""
+    lens = [len(t) for t in token_lists]
+    cu = np.zeros(len(lens) + 1, np.int32)
+    cu[1:] = np.cumsum(lens)
+    input_ids = np.concatenate([np.asarray(t, np.int32) for t in token_lists])
+    positions = np.concatenate([np.arange(n, dtype=np.int32) for n in lens])
+    slots = []
+    for n, table in zip(lens, block_tables):
+        num_blocks = -(-n // block_size)
+        for i in range(num_blocks):
+            start = table[i] * block_size
+            block_len = block_size if i != num_blocks - 1 else n - (num_blocks - 1) * block_size
+            slots.append(np.arange(start, start + block_len, dtype=np.int32))
+    slot_mapping = np.concatenate(slots) if slots else np.zeros(0, np.int32)
+    return input_ids, positions, cu, slot_mapping, max(lens) if lens else 0
 
 
 def advance_decode(next_tokens, input_ids, positions, context: AttentionContext, block_size):
@@ -202,9 +225,19 @@ class DecodeStepRunner:
                                        c.rms_norm_eps, attn.k_cache, attn.v_cache,
                                        context.slot_mapping, c.num_heads, c.num_kv_heads,
                                        c.head_dim)
-                o = paged_attention(q, attn.k_cache, attn.v_cache, context.block_tables,
-                                    context.context_lens, attn.scale, attn.block_size,
-                                    workspace=attn.workspace)
+                if context.is_prefill:
+                    # K/V of the prompt rows were normalised, rotated and stored by
+                    # the fused launch; the prefill kernel wants them packed, so
+                    # they are gathered back from the cache rows just written
+                    flat = (-1, c.num_kv_heads, c.head_dim)
+                    sl = context.slot_mapping.long()
+                    o = variable_length_attention_prefill(
+                        q, attn.k_cache.view(flat)[sl], attn.v_cache.view(flat)[sl],
+                        context.cu_seqlens_q, context.cu_seqlens_k, scale=attn.scale)
+                else:
+                    o = paged_attention(q, attn.k_cache, attn.v_cache, context.block_tables,
+                                        context.context_lens, attn.scale, attn.block_size,
+                                        workspace=attn.workspace)
                 h = F.linear(o.reshape(-1, qs), lw["o"])
                 h, residual = self._rms(h, lw["ln2"], residual)
                 gate, up = F.linear(h, lw["gate_up"]).chunk(2, dim=-1)
@@ -224,7 +257,9 @@ class DecodeStepRunner:
             gate, up = F.linear(h, lw["gate_up"]).chunk(2, dim=-1)
             h = F.linear(F.silu(gate) * up, lw["down"])
         h, _ = self._rms(h, self.final_norm, residual)
-        return F.linear(h, self.embed)                   # logits [T, vocab]
+        if context.is_prefill:                           # only the last token of each prompt
+            h = h[context.last_token_indices.long()]     # (models/qwen3.py:472-491)
+        return F.linear(h, self.embed)                   # logits [T or batch, vocab]
 
     # -- one decode step ------------------------------------------------------
     def make_inputs(self, last_tokens, seq_lens, block_tables):
@@ -233,6 +268,14 @@ class DecodeStepRunner:
         d = self.device
         t = lambda a: torch.from_numpy(a).to(d)
         return t(ids), t(pos), create_decode_context(t(ctx), t(slots), t(bt))
+
+    def make_prefill_inputs(self, token_lists, block_tables):
+        ids, pos, cu, slots, max_len = prepare_prefill(token_lists, block_tables,
+                                                       self.cfg.block_size)
+        d = self.device
+        t = lambda a: torch.from_numpy(a).to(d)
+        cu_t = t(cu)
+        return t(ids), t(pos), create_prefill_context(cu_t, cu_t, max_len, max_len, t(slots))
 
     def step(self, input_ids, positions, context):
         """Eager decode step: logits -> greedy token ids [batch] int64."""

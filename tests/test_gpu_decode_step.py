@@ -186,3 +186,42 @@ def test_generation_graph_matches_host_driven_loop():
         cur_last = want.tolist()
         cur_lens = [n + 1 for n in cur_lens]
     assert ctx.context_lens.cpu().tolist() == cur_lens
+
+
+@pytest.mark.parametrize("fused", [True, False])
+def test_prefill_then_decode_equals_one_longer_prefill(fused):
+    """End to end over every kernel of the path: prefill the prompts (store +
+    prefill attention), decode a few tokens (store + paged decode + metadata),
+    and compare each decode step's logits with a fresh prefill of prompt +
+    generated tokens (its last row sees exactly the same keys)."""
+    print(f"case prefill then decode vs longer prefill fused={fused}", flush=True)
+    cfg, runner = _small_runner(fused)
+    _, check = _small_runner(fused)
+    rng = np.random.Generator(np.random.PCG64(12))
+    lens = [3, 250, 130]
+    prompts = [rng.integers(0, cfg.vocab_size, n).tolist() for n in lens]
+    pages = rng.permutation(cfg.num_kvcache_blocks).tolist()
+    tables, off = [], 0
+    for n in lens:
+        k = -(-(n + 8) // cfg.block_size)
+        tables.append(pages[off:off + k]); off += k
+    ids, pos, ctx = runner.make_prefill_inputs(prompts, tables)
+    logits = runner.forward(ids, pos, ctx).float()
+    assert logits.shape == (len(lens), cfg.vocab_size)
+    seqs = [list(p) for p in prompts]
+    for step in range(4):
+        nxt = logits.argmax(-1).tolist()
+        for s_, t_ in zip(seqs, nxt):
+            s_.append(int(t_))
+        # reference: prefill everything again on a runner with a clean cache
+        c_ids, c_pos, c_ctx = check.make_prefill_inputs(seqs, tables)
+        want = check.forward(c_ids, c_pos, c_ctx).float()
+        # path under test: one decode step on top of the cache built so far
+        used = [t[:-(-len(s_) // cfg.block_size)] for t, s_ in zip(tables, seqs)]
+        d_ids, d_pos, d_ctx = runner.make_inputs(nxt, [len(s_) for s_ in seqs], used)
+        logits = runner.forward(d_ids, d_pos, d_ctx).float()
+        torch.cuda.synchronize()
+        err = (logits - want).abs().max().item()
+        scale = want.abs().max().item()
+        print(f"  step {step}: max |logit diff| {err:.3e} (max |logit| {scale:.2f})", flush=True)
+        assert err <= 0.015 * scale + 0.01
