@@ -70,31 +70,29 @@ struct TileLoader {
   uint32_t row_bytes;   // bytes between consecutive keys
   int last_key, tid, wave, r, qd;
 
-  // Full tiles: uniform 64-bit base (ks rows) + one 32-bit lane offset per
-  // load; the last tile clamps every key to last_key.
+  // One uniform 64-bit base per tile (its first key row) plus one 32-bit lane
+  // offset per load; the last tile clamps every key to last_key.
   __device__ __forceinline__ void issue(int step, uint4& k0, uint4& k1, uint4& v0,
                                         uint4& v1) const {
     const int ks = step * kKeys;
     const uint32_t piece_bytes = (uint32_t)(tid % kPieces) * 16u;
     const int key = tid / kPieces;   // items tid and tid + 256
     const int vk0 = slot_key(wave, 2 * qd), vk1 = slot_key(wave, 2 * qd + 1);
-    if (ks + kKeys - 1 <= last_key) {
-      const char* kb = k_head + (size_t)ks * row_bytes;
-      const char* vb = v_head + (size_t)ks * row_bytes;
-      k0 = *reinterpret_cast<const uint4*>(kb + ((uint32_t)key * row_bytes + piece_bytes));
-      k1 = *reinterpret_cast<const uint4*>(kb + ((uint32_t)(key + 16) * row_bytes + piece_bytes));
-      v0 = *reinterpret_cast<const uint4*>(vb + ((uint32_t)vk0 * row_bytes + (uint32_t)r * 16u));
-      v1 = *reinterpret_cast<const uint4*>(vb + ((uint32_t)vk1 * row_bytes + (uint32_t)r * 16u));
-    } else {
-      k0 = *reinterpret_cast<const uint4*>(
-          k_head + (size_t)min(ks + key, last_key) * row_bytes + piece_bytes);
-      k1 = *reinterpret_cast<const uint4*>(
-          k_head + (size_t)min(ks + key + 16, last_key) * row_bytes + piece_bytes);
-      v0 = *reinterpret_cast<const uint4*>(
-          v_head + (size_t)min(ks + vk0, last_key) * row_bytes + (uint32_t)r * 16u);
-      v1 = *reinterpret_cast<const uint4*>(
-          v_head + (size_t)min(ks + vk1, last_key) * row_bytes + (uint32_t)r * 16u);
+    int a0 = key, a1 = key + 16, b0 = vk0, b1 = vk1;
+    if (ks + kKeys - 1 > last_key) {
+      const int cap = last_key - ks;   // >= 0: the tile starts at a visible key
+      a0 = min(a0, cap);
+      a1 = min(a1, cap);
+      b0 = min(b0, cap);
+      b1 = min(b1, cap);
     }
+    const char* kb = k_head + (size_t)ks * row_bytes;
+    const char* vb = v_head + (size_t)ks * row_bytes;
+    // keys of a tile are < 32 and row_bytes < 2^24 (checked by the host): 24-bit multiplies
+    k0 = *reinterpret_cast<const uint4*>(kb + (__umul24(a0, row_bytes) + piece_bytes));
+    k1 = *reinterpret_cast<const uint4*>(kb + (__umul24(a1, row_bytes) + piece_bytes));
+    v0 = *reinterpret_cast<const uint4*>(vb + (__umul24(b0, row_bytes) + (uint32_t)r * 16u));
+    v1 = *reinterpret_cast<const uint4*>(vb + (__umul24(b1, row_bytes) + (uint32_t)r * 16u));
   }
 
   __device__ __forceinline__ void stage(uint4* k_tile, uint4* vt_tile, const uint4& k0,
@@ -118,6 +116,116 @@ struct TileLoader {
     vt32[base + 7 * dim_stride] = __builtin_amdgcn_perm(v1.w, v0.w, 0x07060302u);
   }
 };
+
+// NaN-propagating maximum: one v_maximum3_f32 per three values, no
+// canonicalising moves on MFMA results.
+__device__ __forceinline__ float max2(float a, float b) {
+  return __builtin_elementwise_maximum(a, b);
+}
+__device__ __forceinline__ float max_of8(const f32x4& a, const f32x4& b) {
+  const float t1 = max2(max2(a[0], a[1]), a[2]);
+  const float t2 = max2(max2(a[3], b[0]), b[1]);
+  return max2(max2(max2(b[2], b[3]), t1), t2);
+}
+
+// One 32-key step of a wave: both column groups (16 query rows each) against
+// the K tile `kt` and the transposed V tile `vt` in LDS.
+//   acc[g][jd]  O^T accumulators, lacc[g] the softmax denominators (every
+//               element of a lane is the sum over all 32 keys of the step, for
+//               the lane's query row: a ones-row times P^T on the matrix core,
+//               from the same bf16 probabilities as the numerator),
+//   m_run[g]    reference point of the exponentials, mneg[g] = -m_run * sl2.
+// MASK: entries beyond `row_limit + 16*g + r` (causal) or `key_limit` (end of
+// the sequence), both relative to the first key of the step, weigh exactly 0.
+template <bool MASK>
+__device__ __forceinline__ void wave_step(const uint4* kt, const uint4* vt,
+                                          const bf16x8 (&qreg)[2][4], f32x4 (&acc)[2][8],
+                                          f32x4 (&lacc)[2], float (&m_run)[2], float (&mneg)[2],
+                                          float sl2, int r, int kg, int row_limit,
+                                          int key_limit) {
+  f32x4 sc[2][2];
+  {
+    bf16x8 ka[2][4];
+#pragma unroll
+    for (int s = 0; s < 4; ++s) {
+      ka[0][s] = as_bf16x8(kt[r * kKRow + 4 * s + kg]);
+      ka[1][s] = as_bf16x8(kt[(16 + r) * kKRow + 4 * s + kg]);
+    }
+#pragma unroll
+    for (int g = 0; g < 2; ++g) {
+      sc[g][0] = sc[g][1] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int s = 0; s < 4; ++s) {
+        sc[g][0] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ka[0][s], qreg[g][s], sc[g][0], 0, 0, 0);
+        sc[g][1] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ka[1][s], qreg[g][s], sc[g][1], 0, 0, 0);
+      }
+    }
+  }
+  bf16x8 va[8];
+#pragma unroll
+  for (int jd = 0; jd < 8; ++jd) va[jd] = as_bf16x8(vt[(jd * 4 + kg) * kPieces + r]);
+  const uint32_t one2 = 0x3F803F80u;   // two bf16 ones
+  const bf16x8 ones = as_bf16x8(make_uint4(one2, one2, one2, one2));
+
+#pragma unroll
+  for (int g = 0; g < 2; ++g) {
+    f32x4& s0 = sc[g][0];
+    f32x4& s1 = sc[g][1];
+    // lane = (query row r of the group, key group kg): keys 4*kg + e and
+    // 16 + 4*kg + e of the step; `limit` = last key of the step the row may see
+    const int limit = MASK ? min(row_limit + 16 * g + r, key_limit) : 0;
+    if (MASK) {
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        if (4 * kg + e > limit) s0[e] = kNegBig;
+        if (16 + 4 * kg + e > limit) s1[e] = kNegBig;
+      }
+    }
+    // Lazy running max: the reference point of the exponentials only moves
+    // when some lane's maximum exceeds it by more than 2^kLazyLog2 (a
+    // wave-uniform decision taken on each lane's own 8 keys, so most steps need
+    // neither a cross-lane reduction nor a rescale of O^T and l).
+    // Probabilities may then exceed 1 (by at most that factor); the final O / l
+    // is unchanged because both carry the same reference.
+    float mx = max_of8(s0, s1);
+    if (__any(fmaf(mx, sl2, mneg[g]) > kLazyLog2)) {
+      mx = max2(mx, __shfl_xor(mx, 16, 64));
+      mx = max2(mx, __shfl_xor(mx, 32, 64));
+      const float m_new = max2(m_run[g], mx);
+      const float alpha = __builtin_amdgcn_exp2f((m_run[g] - m_new) * sl2);
+      m_run[g] = m_new;
+      mneg[g] = -m_new * sl2;
+      lacc[g] *= alpha;
+#pragma unroll
+      for (int jd = 0; jd < 8; ++jd) acc[g][jd] *= alpha;
+    }
+    float p0[4], p1[4];
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      p0[e] = __builtin_amdgcn_exp2f(fmaf(s0[e], sl2, mneg[g]));
+      p1[e] = __builtin_amdgcn_exp2f(fmaf(s1[e], sl2, mneg[g]));
+    }
+    if (MASK) {
+      // masked entries weigh exactly 0 whatever the scale and even for a row
+      // whose reference point is still the initial one
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        if (4 * kg + e > limit) p0[e] = 0.f;
+        if (16 + 4 * kg + e > limit) p1[e] = 0.f;
+      }
+    }
+    uint4 pbits;
+    pbits.x = pack_bf16x2(p0[0], p0[1]);
+    pbits.y = pack_bf16x2(p0[2], p0[3]);
+    pbits.z = pack_bf16x2(p1[0], p1[1]);
+    pbits.w = pack_bf16x2(p1[2], p1[3]);
+    const bf16x8 pb = as_bf16x8(pbits);
+    lacc[g] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ones, pb, lacc[g], 0, 0, 0);
+#pragma unroll
+    for (int jd = 0; jd < 8; ++jd)
+      acc[g][jd] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(va[jd], pb, acc[g][jd], 0, 0, 0);
+  }
+}
 
 struct PrefillArgs {
   const uint4* q;       // [Tq, Hq, 16] pieces
@@ -207,12 +315,14 @@ __global__ __launch_bounds__(kWaves * 64, 2) void prefill_attention_kernel(Prefi
   uint4 kld0, kld1, vld0, vld1;
   const TileLoader ld = {k_head, v_head, row_bytes, k_end - 1, tid, wave, r, kg};
 
-  f32x4 acc[2][8];
-  float m_run[2], l_run[2];
+  const float sl2 = a.scale_log2e;
+  f32x4 acc[2][8], lacc[2];
+  float m_run[2], mneg[2];
 #pragma unroll
   for (int g = 0; g < 2; ++g) {
     m_run[g] = kNegBig;
-    l_run[g] = 0.f;
+    mneg[g] = -kNegBig * sl2;
+    lacc[g] = f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
     for (int jd = 0; jd < 8; ++jd) acc[g][jd] = f32x4{0.f, 0.f, 0.f, 0.f};
   }
@@ -224,113 +334,46 @@ __global__ __launch_bounds__(kWaves * 64, 2) void prefill_attention_kernel(Prefi
   }
   __syncthreads();
 
-  const float sl2 = a.scale_log2e;
   const int wave_row0 = q0 + kRowsPerWave * wave;   // first query row of this wave
 
-  for (int step = 0; step < nsteps; ++step) {
-    const int buf = step & 1;
-    const int ks = step * kKeys;
-    const uint4* kt = k_lds[buf];
-    const uint4* vt = vt_lds[buf];
+  // Steps of this wave, in order: plain ones (every key visible to every row),
+  // masked ones (the diagonal tile, or one that reaches past the last key),
+  // then steps whose keys no row of the wave sees, where it only helps to load.
+  // Three loops rather than a branch inside one keep the accumulators in place.
+  const int n_active = min(nsteps, wave_row0 / kKeys + 1);
+  const int n_plain = min(min(wave_row0, k_end) / kKeys, n_active);
 
-    // the wave has rows that see keys of this step only if its last row >= ks
-    if (wave_row0 + kRowsPerWave - 1 >= ks) {
-      bf16x8 ka[2][4];
-#pragma unroll
-      for (int s = 0; s < 4; ++s) {
-        ka[0][s] = as_bf16x8(kt[r * kKRow + 4 * s + kg]);
-        ka[1][s] = as_bf16x8(kt[(16 + r) * kKRow + 4 * s + kg]);
-      }
-      bf16x8 va[8];
-#pragma unroll
-      for (int jd = 0; jd < 8; ++jd) va[jd] = as_bf16x8(vt[(jd * 4 + kg) * kPieces + r]);
+  // stage the next tile into the other buffer (last read one step ago, before
+  // the previous barrier), fetch the one after it, then meet the others
+#define NVJ_ADVANCE_TILE(step)                                               \
+  do {                                                                       \
+    if ((step) + 1 < nsteps) {                                               \
+      const int nb = ((step) & 1) ^ 1;                                       \
+      ld.stage(k_lds[nb], vt_lds[nb], kld0, kld1, vld0, vld1);               \
+      if ((step) + 2 < nsteps) ld.issue((step) + 2, kld0, kld1, vld0, vld1); \
+    }                                                                        \
+    __syncthreads();                                                         \
+  } while (0)
 
-      // masking is needed where the step reaches past a row of the wave
-      // (diagonal) or past the last key of the sequence
-      const bool need_mask = ks + kKeys - 1 > wave_row0 || ks + kKeys > k_end;
-#pragma unroll
-      for (int g = 0; g < 2; ++g) {
-        f32x4 s0 = {0.f, 0.f, 0.f, 0.f}, s1 = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-        for (int s = 0; s < 4; ++s) {
-          s0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ka[0][s], qreg[g][s], s0, 0, 0, 0);
-          s1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ka[1][s], qreg[g][s], s1, 0, 0, 0);
-        }
-        // lane = (query row, key group): keys ks + 4*kg + e and ks + 16 + 4*kg + e;
-        // `limit` = last key of this step the row may see
-        const int limit = min(wave_row0 + 16 * g + r, k_end - 1) - ks;
-        if (need_mask) {
-#pragma unroll
-          for (int e = 0; e < 4; ++e) {
-            if (4 * kg + e > limit) s0[e] = kNegBig;
-            if (16 + 4 * kg + e > limit) s1[e] = kNegBig;
-          }
-        }
-        float mx = fmaxf(fmaxf(fmaxf(s0[0], s0[1]), fmaxf(s0[2], s0[3])),
-                         fmaxf(fmaxf(s1[0], s1[1]), fmaxf(s1[2], s1[3])));
-        mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
-        mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
-        // Lazy running max: the reference point of the exponentials only moves
-        // when some row's block max exceeds it by more than 2^kLazyLog2 (a
-        // wave-uniform decision), so most steps skip the rescale of O^T and l.
-        // Probabilities may then exceed 1 (by at most that factor); the final
-        // O / l is unchanged because both carry the same reference.
-        const bool move = __any((mx - m_run[g]) * sl2 > kLazyLog2);
-        float mneg = -m_run[g] * sl2;
-        if (move) {
-          const float m_new = fmaxf(m_run[g], mx);
-          const float alpha = __builtin_amdgcn_exp2f((m_run[g] - m_new) * sl2);
-          m_run[g] = m_new;
-          mneg = -m_new * sl2;
-          l_run[g] *= alpha;
-#pragma unroll
-          for (int jd = 0; jd < 8; ++jd) acc[g][jd] *= alpha;
-        }
-        float p0[4], p1[4], psum = 0.f;
-#pragma unroll
-        for (int e = 0; e < 4; ++e) {
-          p0[e] = __builtin_amdgcn_exp2f(fmaf(s0[e], sl2, mneg));
-          p1[e] = __builtin_amdgcn_exp2f(fmaf(s1[e], sl2, mneg));
-        }
-        if (need_mask) {
-          // masked entries weigh exactly 0 whatever the scale and even for a
-          // row whose running max is still the initial one
-#pragma unroll
-          for (int e = 0; e < 4; ++e) {
-            if (4 * kg + e > limit) p0[e] = 0.f;
-            if (16 + 4 * kg + e > limit) p1[e] = 0.f;
-          }
-        }
-#pragma unroll
-        for (int e = 0; e < 4; ++e) psum += p0[e] + p1[e];
-        l_run[g] += psum;
-        uint4 pbits;
-        pbits.x = pack_bf16x2(p0[0], p0[1]);
-        pbits.y = pack_bf16x2(p0[2], p0[3]);
-        pbits.z = pack_bf16x2(p1[0], p1[1]);
-        pbits.w = pack_bf16x2(p1[2], p1[3]);
-        const bf16x8 pb = as_bf16x8(pbits);
-#pragma unroll
-        for (int jd = 0; jd < 8; ++jd)
-          acc[g][jd] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(va[jd], pb, acc[g][jd], 0, 0, 0);
-      }
-    }
-
-    // stage the next tile into the other buffer (last read one step ago, before
-    // the previous barrier), fetch the one after it, then meet the others
-    if (step + 1 < nsteps) {
-      ld.stage(k_lds[buf ^ 1], vt_lds[buf ^ 1], kld0, kld1, vld0, vld1);
-      if (step + 2 < nsteps) ld.issue(step + 2, kld0, kld1, vld0, vld1);
-    }
-    __syncthreads();
+  int step = 0;
+  for (; step < n_plain; ++step) {
+    wave_step<false>(k_lds[step & 1], vt_lds[step & 1], qreg, acc, lacc, m_run, mneg, sl2, r,
+                     kg, 0, 0);
+    NVJ_ADVANCE_TILE(step);
   }
+  for (; step < n_active; ++step) {
+    const int ks = step * kKeys;
+    wave_step<true>(k_lds[step & 1], vt_lds[step & 1], qreg, acc, lacc, m_run, mneg, sl2, r, kg,
+                    wave_row0 - ks, k_end - 1 - ks);
+    NVJ_ADVANCE_TILE(step);
+  }
+  for (; step < nsteps; ++step) NVJ_ADVANCE_TILE(step);
+#undef NVJ_ADVANCE_TILE
 
   // ---- epilogue: acc[g][jd][e] is O[row][dim = 32*kg + 8*e + jd] ----
 #pragma unroll
   for (int g = 0; g < 2; ++g) {
-    float l = l_run[g];
-    l += __shfl_xor(l, 16, 64);
-    l += __shfl_xor(l, 32, 64);
+    const float l = lacc[g][0];   // already summed over every key of the row
     const int row = wave_row0 + 16 * g + r;
     if (row < len_q) {
       const float inv = l > 0.f ? 1.0f / l : 0.f;   // no visible key at all -> zeros
@@ -360,6 +403,7 @@ extern "C" int nvj_prefill_attention_launch(void* stream, const void* q, const v
     return NVJ_ERR_BAD_SHAPE;
   if (num_heads % num_kv_heads != 0) return NVJ_ERR_BAD_SHAPE;
   if (head_dim != kD) return NVJ_ERR_UNSUPPORTED;
+  if (num_kv_heads > 32768) return NVJ_ERR_UNSUPPORTED;   // a key row stays below 2^24 bytes
   if (!(scale >= 0.f)) return NVJ_ERR_BAD_SHAPE;   // the running max assumes a non-negative scale
   if (total_q_tokens == 0 || batch == 0) return NVJ_OK;
   if (!q || !k || !v || !cu_seqlens_q || !cu_seqlens_k || !out) return NVJ_ERR_NULL_POINTER;
