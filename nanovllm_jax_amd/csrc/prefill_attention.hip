@@ -60,9 +60,8 @@ __device__ __forceinline__ int slot_key(int kg, int j) {
 
 // Cooperative tile loads of a workgroup: K 2 pieces per thread, V 2 keys per
 // thread.  K item i of the 512 (key, piece) pairs of a step: key = i / 16,
-// piece = i % 16.  V: wave = key group, lane = (quarter qd = lane >> 4, piece
-// c = lane & 15): the two keys of reduction slots 2*qd and 2*qd + 1 of that key
-// group.  Keys are clamped to the last visible one, so nothing at or beyond
+// piece = i % 16.  V: wave = key group, lane = (slot pair qd, piece r): the two
+// keys of reduction slots 2*qd and 2*qd + 1 of that key group.  Keys are clamped to the last visible one, so nothing at or beyond
 // k_end is read.
 struct TileLoader {
   const char* k_head;   // first key row of the sequence for this kv head
@@ -71,38 +70,44 @@ struct TileLoader {
   int last_key, tid, wave, r, qd;
 
   // One uniform 64-bit base per tile (its first key row) plus one 32-bit lane
-  // offset per load; the last tile clamps every key to last_key.
-  __device__ __forceinline__ void issue(int step, uint4& k0, uint4& k1, uint4& v0,
-                                        uint4& v1) const {
+  // offset per load; the last tile clamps every key to last_key.  Keys of a
+  // tile are < 32 and row_bytes < 2^24 (checked by the host): 24-bit multiplies.
+  __device__ __forceinline__ void issue_k(int step, uint4& k0, uint4& k1) const {
     const int ks = step * kKeys;
     const uint32_t piece_bytes = (uint32_t)(tid % kPieces) * 16u;
-    const int key = tid / kPieces;   // items tid and tid + 256
-    const int vk0 = slot_key(wave, 2 * qd), vk1 = slot_key(wave, 2 * qd + 1);
-    int a0 = key, a1 = key + 16, b0 = vk0, b1 = vk1;
+    int a0 = tid / kPieces, a1 = tid / kPieces + 16;   // items tid and tid + 256
     if (ks + kKeys - 1 > last_key) {
       const int cap = last_key - ks;   // >= 0: the tile starts at a visible key
       a0 = min(a0, cap);
       a1 = min(a1, cap);
+    }
+    const char* kb = k_head + (size_t)ks * row_bytes;
+    k0 = *reinterpret_cast<const uint4*>(kb + (__umul24(a0, row_bytes) + piece_bytes));
+    k1 = *reinterpret_cast<const uint4*>(kb + (__umul24(a1, row_bytes) + piece_bytes));
+  }
+
+  __device__ __forceinline__ void issue_v(int step, uint4& v0, uint4& v1) const {
+    const int ks = step * kKeys;
+    int b0 = slot_key(wave, 2 * qd), b1 = slot_key(wave, 2 * qd + 1);
+    if (ks + kKeys - 1 > last_key) {
+      const int cap = last_key - ks;
       b0 = min(b0, cap);
       b1 = min(b1, cap);
     }
-    const char* kb = k_head + (size_t)ks * row_bytes;
     const char* vb = v_head + (size_t)ks * row_bytes;
-    // keys of a tile are < 32 and row_bytes < 2^24 (checked by the host): 24-bit multiplies
-    k0 = *reinterpret_cast<const uint4*>(kb + (__umul24(a0, row_bytes) + piece_bytes));
-    k1 = *reinterpret_cast<const uint4*>(kb + (__umul24(a1, row_bytes) + piece_bytes));
     v0 = *reinterpret_cast<const uint4*>(vb + (__umul24(b0, row_bytes) + (uint32_t)r * 16u));
     v1 = *reinterpret_cast<const uint4*>(vb + (__umul24(b1, row_bytes) + (uint32_t)r * 16u));
   }
 
-  __device__ __forceinline__ void stage(uint4* k_tile, uint4* vt_tile, const uint4& k0,
-                                        const uint4& k1, const uint4& v0,
-                                        const uint4& v1) const {
+  __device__ __forceinline__ void stage_k(uint4* k_tile, const uint4& k0, const uint4& k1) const {
     const int piece = tid % kPieces, key = tid / kPieces;
     k_tile[key * kKRow + piece] = k0;
     k_tile[(key + 16) * kKRow + piece] = k1;
-    // 2 keys x 8 dims -> per dim the (key0, key1) pair, at slot pair 2*qd of the
-    // operand of (dim jd, key group = wave, piece r)
+  }
+
+  // 2 keys x 8 dims -> per dim the (key0, key1) pair, at slot pair 2*qd of the
+  // operand of (dim jd, key group = wave, piece r)
+  __device__ __forceinline__ void stage_v(uint4* vt_tile, const uint4& v0, const uint4& v1) const {
     uint32_t* vt32 = reinterpret_cast<uint32_t*>(vt_tile);
     const int base = (wave * kPieces + r) * 4 + qd;
     const int dim_stride = 4 * kPieces * 4;   // dwords between consecutive jd
@@ -128,51 +133,67 @@ __device__ __forceinline__ float max_of8(const f32x4& a, const f32x4& b) {
   return max2(max2(max2(b[2], b[3]), t1), t2);
 }
 
-// One 32-key step of a wave: both column groups (16 query rows each) against
-// the K tile `kt` and the transposed V tile `vt` in LDS.
-//   acc[g][jd]  O^T accumulators, lacc[g] the softmax denominators (every
-//               element of a lane is the sum over all 32 keys of the step, for
-//               the lane's query row: a ones-row times P^T on the matrix core,
-//               from the same bf16 probabilities as the numerator),
-//   m_run[g]    reference point of the exponentials, mneg[g] = -m_run * sl2.
-// MASK: entries beyond `row_limit + 16*g + r` (causal) or `key_limit` (end of
-// the sequence), both relative to the first key of the step, weigh exactly 0.
-template <bool MASK>
-__device__ __forceinline__ void wave_step(const uint4* kt, const uint4* vt,
-                                          const bf16x8 (&qreg)[2][4], f32x4 (&acc)[2][8],
-                                          f32x4 (&lacc)[2], float (&m_run)[2], float (&mneg)[2],
-                                          float sl2, int r, int kg, int row_limit,
-                                          int key_limit) {
-  f32x4 sc[2][2];
-  {
-    bf16x8 ka[2][4];
+// S^T of one 32-key tile against both column groups (16 query rows each):
+// sc[g][h] holds keys 16*h + 4*kg + e of the tile for query row r of group g.
+__device__ __forceinline__ void scores_of_tile(const uint4* kt, const bf16x8 (&qreg)[2][4],
+                                               f32x4 (&sc)[2][2], int r, int kg) {
+  bf16x8 ka[2][4];
+#pragma unroll
+  for (int s = 0; s < 4; ++s) {
+    ka[0][s] = as_bf16x8(kt[r * kKRow + 4 * s + kg]);
+    ka[1][s] = as_bf16x8(kt[(16 + r) * kKRow + 4 * s + kg]);
+  }
+#pragma unroll
+  for (int g = 0; g < 2; ++g) {
+    sc[g][0] = sc[g][1] = f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
     for (int s = 0; s < 4; ++s) {
-      ka[0][s] = as_bf16x8(kt[r * kKRow + 4 * s + kg]);
-      ka[1][s] = as_bf16x8(kt[(16 + r) * kKRow + 4 * s + kg]);
-    }
-#pragma unroll
-    for (int g = 0; g < 2; ++g) {
-      sc[g][0] = sc[g][1] = f32x4{0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-      for (int s = 0; s < 4; ++s) {
-        sc[g][0] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ka[0][s], qreg[g][s], sc[g][0], 0, 0, 0);
-        sc[g][1] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ka[1][s], qreg[g][s], sc[g][1], 0, 0, 0);
-      }
+      sc[g][0] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ka[0][s], qreg[g][s], sc[g][0], 0, 0, 0);
+      sc[g][1] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ka[1][s], qreg[g][s], sc[g][1], 0, 0, 0);
     }
   }
+}
+
+// O^T += V^T . P^T and l += 1 . P^T for the probabilities `pb` of one tile whose
+// transposed V is `vt`.  Every element of lacc[g] of a lane is the sum over all
+// 32 keys of the tile for the lane's query row: a ones-row times P^T on the
+// matrix core, from the same bf16 probabilities as the numerator.
+__device__ __forceinline__ void accumulate_tile(const uint4* vt, const bf16x8 (&pb)[2],
+                                                f32x4 (&acc)[2][8], f32x4 (&lacc)[2], int r,
+                                                int kg) {
   bf16x8 va[8];
 #pragma unroll
   for (int jd = 0; jd < 8; ++jd) va[jd] = as_bf16x8(vt[(jd * 4 + kg) * kPieces + r]);
   const uint32_t one2 = 0x3F803F80u;   // two bf16 ones
   const bf16x8 ones = as_bf16x8(make_uint4(one2, one2, one2, one2));
+#pragma unroll
+  for (int g = 0; g < 2; ++g) {
+    lacc[g] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ones, pb[g], lacc[g], 0, 0, 0);
+#pragma unroll
+    for (int jd = 0; jd < 8; ++jd)
+      acc[g][jd] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(va[jd], pb[g], acc[g][jd], 0, 0, 0);
+  }
+}
 
+// Probabilities of one tile from its scores (fp32 online softmax on the
+// accumulator layout), already in B-operand layout.
+//   m_run[g]  reference point of the exponentials, mneg[g] = -m_run * sl2.
+// MASK: entries beyond `row_limit + 16*g + r` (causal) or `key_limit` (end of
+// the sequence), both relative to the first key of the tile, weigh exactly 0.
+// Must run after the previous tile has been accumulated: moving the reference
+// point rescales acc and lacc.
+template <bool MASK>
+__device__ __forceinline__ void probabilities_of_tile(f32x4 (&sc)[2][2], bf16x8 (&pb)[2],
+                                                      f32x4 (&acc)[2][8], f32x4 (&lacc)[2],
+                                                      float (&m_run)[2], float (&mneg)[2],
+                                                      float sl2, int r, int kg, int row_limit,
+                                                      int key_limit) {
 #pragma unroll
   for (int g = 0; g < 2; ++g) {
     f32x4& s0 = sc[g][0];
     f32x4& s1 = sc[g][1];
     // lane = (query row r of the group, key group kg): keys 4*kg + e and
-    // 16 + 4*kg + e of the step; `limit` = last key of the step the row may see
+    // 16 + 4*kg + e of the tile; `limit` = last key of the tile the row may see
     const int limit = MASK ? min(row_limit + 16 * g + r, key_limit) : 0;
     if (MASK) {
 #pragma unroll
@@ -183,7 +204,7 @@ __device__ __forceinline__ void wave_step(const uint4* kt, const uint4* vt,
     }
     // Lazy running max: the reference point of the exponentials only moves
     // when some lane's maximum exceeds it by more than 2^kLazyLog2 (a
-    // wave-uniform decision taken on each lane's own 8 keys, so most steps need
+    // wave-uniform decision taken on each lane's own 8 keys, so most tiles need
     // neither a cross-lane reduction nor a rescale of O^T and l).
     // Probabilities may then exceed 1 (by at most that factor); the final O / l
     // is unchanged because both carry the same reference.
@@ -219,11 +240,7 @@ __device__ __forceinline__ void wave_step(const uint4* kt, const uint4* vt,
     pbits.y = pack_bf16x2(p0[2], p0[3]);
     pbits.z = pack_bf16x2(p1[0], p1[1]);
     pbits.w = pack_bf16x2(p1[2], p1[3]);
-    const bf16x8 pb = as_bf16x8(pbits);
-    lacc[g] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ones, pb, lacc[g], 0, 0, 0);
-#pragma unroll
-    for (int jd = 0; jd < 8; ++jd)
-      acc[g][jd] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(va[jd], pb, acc[g][jd], 0, 0, 0);
+    pb[g] = as_bf16x8(pbits);
   }
 }
 
@@ -313,7 +330,10 @@ __global__ __launch_bounds__(kWaves * 64, 2) void prefill_attention_kernel(Prefi
       reinterpret_cast<const char*>(a.v + ((int64_t)k_base * a.num_kv_heads + kvh) * kPieces);
 
   uint4 kld0, kld1, vld0, vld1;
-  const TileLoader ld = {k_head, v_head, row_bytes, k_end - 1, tid, wave, r, kg};
+  // V is loaded by lane = (piece low 3 bits, slot pair qd, piece high bit): the
+  // first 32 lanes then write 8 pieces x 4 slot pairs = 32 different LDS banks
+  const TileLoader ld = {k_head, v_head, row_bytes, k_end - 1, tid, wave,
+                         (lane & 7) | ((lane >> 5) << 3), (lane >> 3) & 3};
 
   const float sl2 = a.scale_log2e;
   f32x4 acc[2][8], lacc[2];
@@ -327,48 +347,74 @@ __global__ __launch_bounds__(kWaves * 64, 2) void prefill_attention_kernel(Prefi
     for (int jd = 0; jd < 8; ++jd) acc[g][jd] = f32x4{0.f, 0.f, 0.f, 0.f};
   }
 
+  // Software pipeline over the tiles: iteration i computes the scores of tile i
+  // on the matrix core, then accumulates tile i-1 (probabilities kept from the
+  // previous iteration) while the vector ALU turns the scores of tile i into
+  // probabilities.  So K of tile i and V^T of tile i-1 are read in iteration i:
+  // the K buffers run one tile ahead of the V^T buffers.  At the top of
+  // iteration i the staging registers hold K of tile i+1 and V of tile i.
+  const int wave_row0 = q0 + kRowsPerWave * wave;   // first query row of this wave
+  {
+    // V^T "of tile -1" (probabilities are zero there, but 0 * NaN is not 0)
+    const uint4 zero = make_uint4(0u, 0u, 0u, 0u);
+    vt_lds[1][tid] = zero;
+    vt_lds[1][tid + kWaves * 64] = zero;
+  }
   if (nsteps > 0) {
-    ld.issue(0, kld0, kld1, vld0, vld1);
-    ld.stage(k_lds[0], vt_lds[0], kld0, kld1, vld0, vld1);
-    if (nsteps > 1) ld.issue(1, kld0, kld1, vld0, vld1);
+    ld.issue_k(0, kld0, kld1);
+    ld.issue_v(0, vld0, vld1);
+    ld.stage_k(k_lds[0], kld0, kld1);
+    if (nsteps > 1) ld.issue_k(1, kld0, kld1);
   }
   __syncthreads();
 
-  const int wave_row0 = q0 + kRowsPerWave * wave;   // first query row of this wave
-
-  // Steps of this wave, in order: plain ones (every key visible to every row),
+  // Tiles of this wave, in order: plain ones (every key visible to every row),
   // masked ones (the diagonal tile, or one that reaches past the last key),
-  // then steps whose keys no row of the wave sees, where it only helps to load.
-  // Three loops rather than a branch inside one keep the accumulators in place.
+  // then tiles whose keys no row of the wave sees, where it only helps to load.
+  // Separate loops rather than a branch inside one keep the accumulators in place.
   const int n_active = min(nsteps, wave_row0 / kKeys + 1);
   const int n_plain = min(min(wave_row0, k_end) / kKeys, n_active);
 
-  // stage the next tile into the other buffer (last read one step ago, before
-  // the previous barrier), fetch the one after it, then meet the others
-#define NVJ_ADVANCE_TILE(step)                                               \
-  do {                                                                       \
-    if ((step) + 1 < nsteps) {                                               \
-      const int nb = ((step) & 1) ^ 1;                                       \
-      ld.stage(k_lds[nb], vt_lds[nb], kld0, kld1, vld0, vld1);               \
-      if ((step) + 2 < nsteps) ld.issue((step) + 2, kld0, kld1, vld0, vld1); \
-    }                                                                        \
-    __syncthreads();                                                         \
+  // Stage V^T of tile i and K of tile i+1 (their buffers were last read one
+  // iteration ago, before the previous barrier) and fetch the tiles after them.
+#define NVJ_STAGE_TILES(i)                                        \
+  do {                                                            \
+    ld.stage_v(vt_lds[(i) & 1], vld0, vld1);                      \
+    if ((i) + 1 < nsteps) {                                       \
+      ld.stage_k(k_lds[((i) + 1) & 1], kld0, kld1);               \
+      ld.issue_v((i) + 1, vld0, vld1);                            \
+      if ((i) + 2 < nsteps) ld.issue_k((i) + 2, kld0, kld1);      \
+    }                                                             \
   } while (0)
 
-  int step = 0;
-  for (; step < n_plain; ++step) {
-    wave_step<false>(k_lds[step & 1], vt_lds[step & 1], qreg, acc, lacc, m_run, mneg, sl2, r,
-                     kg, 0, 0);
-    NVJ_ADVANCE_TILE(step);
+  f32x4 sc[2][2];
+  bf16x8 pb[2];
+  pb[0] = pb[1] = as_bf16x8(make_uint4(0u, 0u, 0u, 0u));
+  int i = 0;
+  for (; i < n_plain; ++i) {
+    scores_of_tile(k_lds[i & 1], qreg, sc, r, kg);
+    NVJ_STAGE_TILES(i);
+    accumulate_tile(vt_lds[(i & 1) ^ 1], pb, acc, lacc, r, kg);
+    probabilities_of_tile<false>(sc, pb, acc, lacc, m_run, mneg, sl2, r, kg, 0, 0);
+    __syncthreads();
   }
-  for (; step < n_active; ++step) {
-    const int ks = step * kKeys;
-    wave_step<true>(k_lds[step & 1], vt_lds[step & 1], qreg, acc, lacc, m_run, mneg, sl2, r, kg,
-                    wave_row0 - ks, k_end - 1 - ks);
-    NVJ_ADVANCE_TILE(step);
+  for (; i < n_active; ++i) {
+    const int ks = i * kKeys;
+    scores_of_tile(k_lds[i & 1], qreg, sc, r, kg);
+    NVJ_STAGE_TILES(i);
+    accumulate_tile(vt_lds[(i & 1) ^ 1], pb, acc, lacc, r, kg);
+    probabilities_of_tile<true>(sc, pb, acc, lacc, m_run, mneg, sl2, r, kg, wave_row0 - ks,
+                                k_end - 1 - ks);
+    __syncthreads();
   }
-  for (; step < nsteps; ++step) NVJ_ADVANCE_TILE(step);
-#undef NVJ_ADVANCE_TILE
+  // the last tile of the wave is still to be accumulated; its V^T stays in
+  // place until the staging of the iteration after this one
+  if (n_active > 0) accumulate_tile(vt_lds[(n_active - 1) & 1], pb, acc, lacc, r, kg);
+  for (; i < nsteps; ++i) {
+    NVJ_STAGE_TILES(i);
+    __syncthreads();
+  }
+#undef NVJ_STAGE_TILES
 
   // ---- epilogue: acc[g][jd][e] is O[row][dim = 32*kg + 8*e + jd] ----
 #pragma unroll
