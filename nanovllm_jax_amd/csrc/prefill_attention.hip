@@ -11,17 +11,23 @@
 //
 // MFMA-bound.  One workgroup = 4 waves = 128 query rows of one (sequence, query
 // head); a wave owns 32 rows as two groups of 16 MFMA columns.  Keys are walked
-// 32 at a time; the K tile and the V tile of a step are fetched once per
-// workgroup and staged in LDS (double-buffered, one barrier per step):
-//   * K as rows of 16-byte pieces (padded), read back as the A operand of
+// 32 at a time.  The K rows and the V rows of a tile go from global memory
+// straight into LDS (global_load_lds_dwordx4: no staging registers, no LDS
+// write instructions), row-major with the 16-byte pieces of a row permuted so
+// that the reads below are free of bank conflicts, in rings of 3 (K) and 4 (V)
+// tiles fetched two tiles ahead; one barrier per tile:
+//   * K is read back with ds_read_b128 as the A operand of
 //     S^T[key, q] = K . Q^T  (v_mfma_f32_16x16x32_bf16, Q^T of both groups in
 //     registers for the whole tile);
-//   * V already transposed into A operands of O^T[dim, q] += V^T . P^T: the
-//     loading lane holds 2 keys x 8 dims and writes, per dim, the 2-key pair
-//     where the operand of (dim group, key group) expects it.
+//   * V is read back with the transposing LDS read (ds_read_b64_tr_b16), which
+//     hands each lane four keys of one head dimension: the A operand of
+//     O^T[dim, q] += V^T . P^T.
 // Softmax is the fp32 online form on the accumulator layout; P^T comes out of
 // the S^T accumulators already in B-operand layout (same reduction-slot <-> key
 // map as the decode kernel).  Only tiles that touch the diagonal are masked.
+// The loop is software-pipelined: the scores of tile i are issued to the matrix
+// core, then tile i-1 is accumulated while the vector ALU turns the scores of
+// tile i into probabilities.
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
@@ -38,7 +44,9 @@ constexpr int kBM = 128;             // query rows per workgroup
 constexpr int kWaves = 4;
 constexpr int kRowsPerWave = kBM / kWaves;   // 32 = two column groups of 16
 constexpr int kKeys = 32;            // keys per step
-constexpr int kKRow = kPieces + 1;   // padded K row in LDS, in pieces
+constexpr int kTileBytes = kKeys * kD * 2;   // one K or V tile in LDS: 32 rows of 256 bytes
+constexpr int kKStages = 3;          // K tiles i .. i+2 are live in iteration i
+constexpr int kVStages = 4;          // V tiles i-1 .. i+2
 constexpr float kNegBig = -1.0e30f;
 constexpr float kLazyLog2 = 8.0f;    // running max moves only for gains above 2^8
 constexpr float kLog2e = 1.4426950408889634f;
@@ -58,69 +66,75 @@ __device__ __forceinline__ int slot_key(int kg, int j) {
   return j < 4 ? 4 * kg + j : 16 + 4 * kg + (j - 4);
 }
 
-// Cooperative tile loads of a workgroup: K 2 pieces per thread, V 2 keys per
-// thread.  K item i of the 512 (key, piece) pairs of a step: key = i / 16,
-// piece = i % 16.  V: wave = key group, lane = (slot pair qd, piece r): the two
-// keys of reduction slots 2*qd and 2*qd + 1 of that key group.  Keys are clamped to the last visible one, so nothing at or beyond
+typedef __attribute__((address_space(3))) char* lds_ptr;
+typedef __attribute__((ext_vector_type(4))) __bf16 bf16x4;
+
+// LDS layout of a tile: row R (key R of the tile) at byte 256 * R, its 16-byte
+// piece p at position p ^ (R & 15) for K and p ^ (2 * (R & 7)) for V.
+//   K read (ds_read_b128): the 16 lanes of a key group read one piece of 16
+//     different rows -> 16 different positions.
+//   V read (ds_read_b64_tr_b16): the 16 lanes of a key group read four 8-byte
+//     chunks of each of 4 rows -> 16 different 8-byte slots modulo 128 bytes.
+__device__ __forceinline__ int k_position(int row, int piece) { return piece ^ (row & 15); }
+__device__ __forceinline__ int v_position(int row, int piece) { return piece ^ (2 * (row & 7)); }
+
+// One 16-byte global -> LDS copy per lane: lane l's piece lands at
+// lds_base + 16 * l (lds_base wave-uniform), fetched from base + offset.
+// Counts in vmcnt like any load; the compiler does not see it as one, so the
+// waits are written out by hand (wait_tiles_in_flight).
+__device__ __forceinline__ void copy16_to_lds(const char* base, uint32_t offset,
+                                              uint32_t lds_base) {
+  asm volatile(
+      "s_mov_b32 m0, %0\n\t"
+      "s_nop 0\n\t"
+      "global_load_lds_dwordx4 %1, %2"
+      :
+      : "s"(lds_base), "v"(offset), "s"(base)
+      : "memory");
+}
+
+// Cooperative tile copies of a workgroup.  A tile is 512 pieces of K and 512 of
+// V; wave w copies rows 8w .. 8w+7 of both with two instructions each (4 rows =
+// 1024 contiguous LDS bytes per instruction).  Lane l of instruction j writes
+// position l % 16 of row 8w + 4j + l / 16 and fetches the piece that belongs
+// there.  Rows are clamped to the last visible key, so nothing at or beyond
 // k_end is read.
-struct TileLoader {
+struct TileCopier {
   const char* k_head;   // first key row of the sequence for this kv head
   const char* v_head;
-  uint32_t row_bytes;   // bytes between consecutive keys
-  int last_key, tid, wave, r, qd;
+  uint32_t row_bytes;   // bytes between consecutive keys; < 2^24 (checked by the host)
+  uint32_t k_lds, v_lds;   // LDS byte addresses of the two rings
+  int last_key, last_tile, wave, lane;
 
-  // One uniform 64-bit base per tile (its first key row) plus one 32-bit lane
-  // offset per load; the last tile clamps every key to last_key.  Keys of a
-  // tile are < 32 and row_bytes < 2^24 (checked by the host): 24-bit multiplies.
-  __device__ __forceinline__ void issue_k(int step, uint4& k0, uint4& k1) const {
-    const int ks = step * kKeys;
-    const uint32_t piece_bytes = (uint32_t)(tid % kPieces) * 16u;
-    int a0 = tid / kPieces, a1 = tid / kPieces + 16;   // items tid and tid + 256
-    if (ks + kKeys - 1 > last_key) {
-      const int cap = last_key - ks;   // >= 0: the tile starts at a visible key
-      a0 = min(a0, cap);
-      a1 = min(a1, cap);
-    }
+  __device__ __forceinline__ void issue(int tile, int k_stage, int v_stage) const {
+    tile = min(tile, last_tile);   // past the end: fetch the last tile again (same instruction count)
+    const int ks = tile * kKeys;
+    const int cap = last_key - ks;   // >= 0: a tile starts at a visible key
     const char* kb = k_head + (size_t)ks * row_bytes;
-    k0 = *reinterpret_cast<const uint4*>(kb + (__umul24(a0, row_bytes) + piece_bytes));
-    k1 = *reinterpret_cast<const uint4*>(kb + (__umul24(a1, row_bytes) + piece_bytes));
-  }
-
-  __device__ __forceinline__ void issue_v(int step, uint4& v0, uint4& v1) const {
-    const int ks = step * kKeys;
-    int b0 = slot_key(wave, 2 * qd), b1 = slot_key(wave, 2 * qd + 1);
-    if (ks + kKeys - 1 > last_key) {
-      const int cap = last_key - ks;
-      b0 = min(b0, cap);
-      b1 = min(b1, cap);
-    }
     const char* vb = v_head + (size_t)ks * row_bytes;
-    v0 = *reinterpret_cast<const uint4*>(vb + (__umul24(b0, row_bytes) + (uint32_t)r * 16u));
-    v1 = *reinterpret_cast<const uint4*>(vb + (__umul24(b1, row_bytes) + (uint32_t)r * 16u));
-  }
-
-  __device__ __forceinline__ void stage_k(uint4* k_tile, const uint4& k0, const uint4& k1) const {
-    const int piece = tid % kPieces, key = tid / kPieces;
-    k_tile[key * kKRow + piece] = k0;
-    k_tile[(key + 16) * kKRow + piece] = k1;
-  }
-
-  // 2 keys x 8 dims -> per dim the (key0, key1) pair, at slot pair 2*qd of the
-  // operand of (dim jd, key group = wave, piece r)
-  __device__ __forceinline__ void stage_v(uint4* vt_tile, const uint4& v0, const uint4& v1) const {
-    uint32_t* vt32 = reinterpret_cast<uint32_t*>(vt_tile);
-    const int base = (wave * kPieces + r) * 4 + qd;
-    const int dim_stride = 4 * kPieces * 4;   // dwords between consecutive jd
-    vt32[base + 0 * dim_stride] = __builtin_amdgcn_perm(v1.x, v0.x, 0x05040100u);
-    vt32[base + 1 * dim_stride] = __builtin_amdgcn_perm(v1.x, v0.x, 0x07060302u);
-    vt32[base + 2 * dim_stride] = __builtin_amdgcn_perm(v1.y, v0.y, 0x05040100u);
-    vt32[base + 3 * dim_stride] = __builtin_amdgcn_perm(v1.y, v0.y, 0x07060302u);
-    vt32[base + 4 * dim_stride] = __builtin_amdgcn_perm(v1.z, v0.z, 0x05040100u);
-    vt32[base + 5 * dim_stride] = __builtin_amdgcn_perm(v1.z, v0.z, 0x07060302u);
-    vt32[base + 6 * dim_stride] = __builtin_amdgcn_perm(v1.w, v0.w, 0x05040100u);
-    vt32[base + 7 * dim_stride] = __builtin_amdgcn_perm(v1.w, v0.w, 0x07060302u);
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+      const int row = 8 * wave + 4 * j + (lane >> 4);
+      const uint32_t row_off = __umul24(min(row, cap), row_bytes);
+      const uint32_t dst = (uint32_t)(2 * wave + j) * 1024u;
+      copy16_to_lds(kb, row_off + 16u * k_position(row, lane & 15),
+                    k_lds + (uint32_t)k_stage * kTileBytes + dst);
+      copy16_to_lds(vb, row_off + 16u * v_position(row, lane & 15),
+                    v_lds + (uint32_t)v_stage * kTileBytes + dst);
+    }
   }
 };
+constexpr int kCopiesPerTile = 4;   // copy16_to_lds calls of one lane per tile
+
+// Blocks until at most `tiles` of this lane's most recent tile copies are still
+// in flight (vmcnt counts the copies in order).
+template <int TILES>
+__device__ __forceinline__ void wait_tiles_in_flight() {
+  static_assert(TILES == 0 || TILES == 1, "vmcnt immediates below");
+  if (TILES == 0) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  else asm volatile("s_waitcnt vmcnt(4)" ::: "memory");
+  static_assert(kCopiesPerTile == 4, "vmcnt immediates above");
+}
 
 // NaN-propagating maximum: one v_maximum3_f32 per three values, no
 // canonicalising moves on MFMA results.
@@ -135,13 +149,15 @@ __device__ __forceinline__ float max_of8(const f32x4& a, const f32x4& b) {
 
 // S^T of one 32-key tile against both column groups (16 query rows each):
 // sc[g][h] holds keys 16*h + 4*kg + e of the tile for query row r of group g.
-__device__ __forceinline__ void scores_of_tile(const uint4* kt, const bf16x8 (&qreg)[2][4],
+__device__ __forceinline__ void scores_of_tile(lds_ptr kt, const bf16x8 (&qreg)[2][4],
                                                f32x4 (&sc)[2][2], int r, int kg) {
   bf16x8 ka[2][4];
 #pragma unroll
   for (int s = 0; s < 4; ++s) {
-    ka[0][s] = as_bf16x8(kt[r * kKRow + 4 * s + kg]);
-    ka[1][s] = as_bf16x8(kt[(16 + r) * kKRow + 4 * s + kg]);
+    // rows r and 16 + r share a position: (16 + r) & 15 == r
+    const int at = 256 * r + 16 * k_position(r, 4 * s + kg);
+    ka[0][s] = *reinterpret_cast<const __attribute__((address_space(3))) bf16x8*>(kt + at);
+    ka[1][s] = *reinterpret_cast<const __attribute__((address_space(3))) bf16x8*>(kt + at + 16 * 256);
   }
 #pragma unroll
   for (int g = 0; g < 2; ++g) {
@@ -155,15 +171,31 @@ __device__ __forceinline__ void scores_of_tile(const uint4* kt, const bf16x8 (&q
 }
 
 // O^T += V^T . P^T and l += 1 . P^T for the probabilities `pb` of one tile whose
-// transposed V is `vt`.  Every element of lacc[g] of a lane is the sum over all
-// 32 keys of the tile for the lane's query row: a ones-row times P^T on the
-// matrix core, from the same bf16 probabilities as the numerator.
-__device__ __forceinline__ void accumulate_tile(const uint4* vt, const bf16x8 (&pb)[2],
+// V rows are at `vt`.  Operand jd covers head dimensions 16*jd .. 16*jd + 15.
+// ds_read_b64_tr_b16 works on groups of 16 lanes: source lane s = 4a + b of a
+// group points at 4 consecutive bf16 (b selects which 4 of the 16 dimensions)
+// of row a; result lane 4b + j receives, as element a, the j-th of those from
+// source lane 4a + b.  With row a = key 4*kg + a of the tile (then 16 + 4*kg + a
+// for the second read) lane i of the group ends up with keys of reduction
+// slots 0..3 (then 4..7) of dimension 16*jd + i: the A operand.
+// Every element of lacc[g] of a lane is the sum over all 32 keys of the tile for
+// the lane's query row: a ones-row times P^T on the matrix core, from the same
+// bf16 probabilities as the numerator.
+__device__ __forceinline__ void accumulate_tile(lds_ptr vt, const bf16x8 (&pb)[2],
                                                 f32x4 (&acc)[2][8], f32x4 (&lacc)[2], int r,
                                                 int kg) {
+  const int row = 4 * kg + (r >> 2);   // (16 + row) & 7 == row & 7: both reads share positions
+  const int chunk = r & 3;             // 8-byte chunk of the 32 bytes of a dimension group
   bf16x8 va[8];
 #pragma unroll
-  for (int jd = 0; jd < 8; ++jd) va[jd] = as_bf16x8(vt[(jd * 4 + kg) * kPieces + r]);
+  for (int jd = 0; jd < 8; ++jd) {
+    const int at = 256 * row + 16 * v_position(row, 2 * jd + (chunk >> 1)) + 8 * (chunk & 1);
+    const bf16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4bf16(
+        reinterpret_cast<__attribute__((address_space(3))) bf16x4*>(vt + at));
+    const bf16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4bf16(
+        reinterpret_cast<__attribute__((address_space(3))) bf16x4*>(vt + at + 16 * 256));
+    va[jd] = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+  }
   const uint32_t one2 = 0x3F803F80u;   // two bf16 ones
   const bf16x8 ones = as_bf16x8(make_uint4(one2, one2, one2, one2));
 #pragma unroll
@@ -258,8 +290,8 @@ struct PrefillArgs {
 // grid.x = 8 * ceil(tile bound * Hq / 8) workgroups (see the work-item mapping below).
 __global__ __launch_bounds__(kWaves * 64, 2) void prefill_attention_kernel(PrefillArgs a,
                                                                         int num_tiles_bound) {
-  __shared__ uint4 k_lds[2][kKeys * kKRow];
-  __shared__ uint4 vt_lds[2][8 * 4 * kPieces];   // [dim-in-piece jd][key group][piece]
+  __shared__ uint4 k_ring[kKStages * kTileBytes / 16];
+  __shared__ uint4 v_ring[kVStages * kTileBytes / 16];
 
   const int tid = threadIdx.x;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -329,11 +361,10 @@ __global__ __launch_bounds__(kWaves * 64, 2) void prefill_attention_kernel(Prefi
   const char* v_head =
       reinterpret_cast<const char*>(a.v + ((int64_t)k_base * a.num_kv_heads + kvh) * kPieces);
 
-  uint4 kld0, kld1, vld0, vld1;
-  // V is loaded by lane = (piece low 3 bits, slot pair qd, piece high bit): the
-  // first 32 lanes then write 8 pieces x 4 slot pairs = 32 different LDS banks
-  const TileLoader ld = {k_head, v_head, row_bytes, k_end - 1, tid, wave,
-                         (lane & 7) | ((lane >> 5) << 3), (lane >> 3) & 3};
+  const lds_ptr k_lds = (lds_ptr)k_ring;
+  const lds_ptr v_lds = (lds_ptr)v_ring;
+  const TileCopier copier = {k_head, v_head, row_bytes, (uint32_t)(uintptr_t)k_lds,
+                             (uint32_t)(uintptr_t)v_lds, k_end - 1, nsteps - 1, wave, lane};
 
   const float sl2 = a.scale_log2e;
   f32x4 acc[2][8], lacc[2];
@@ -347,91 +378,87 @@ __global__ __launch_bounds__(kWaves * 64, 2) void prefill_attention_kernel(Prefi
     for (int jd = 0; jd < 8; ++jd) acc[g][jd] = f32x4{0.f, 0.f, 0.f, 0.f};
   }
 
-  // Software pipeline over the tiles: iteration i computes the scores of tile i
-  // on the matrix core, then accumulates tile i-1 (probabilities kept from the
+  // Software pipeline over the tiles: iteration i issues the scores of tile i to
+  // the matrix core, then accumulates tile i-1 (probabilities kept from the
   // previous iteration) while the vector ALU turns the scores of tile i into
-  // probabilities.  So K of tile i and V^T of tile i-1 are read in iteration i:
-  // the K buffers run one tile ahead of the V^T buffers.  At the top of
-  // iteration i the staging registers hold K of tile i+1 and V of tile i.
+  // probabilities.  Iteration i therefore reads K of tile i and V of tile i-1,
+  // and starts the copies of tile i+2 into the ring slots last read in iteration
+  // i-1 (K of tile i-1, V of tile i-2).  Before the barrier that ends it, every
+  // lane waits for its copies of tile i+1.
   const int wave_row0 = q0 + kRowsPerWave * wave;   // first query row of this wave
-  {
-    // V^T "of tile -1" (probabilities are zero there, but 0 * NaN is not 0)
-    const uint4 zero = make_uint4(0u, 0u, 0u, 0u);
-    vt_lds[1][tid] = zero;
-    vt_lds[1][tid + kWaves * 64] = zero;
-  }
   if (nsteps > 0) {
-    ld.issue_k(0, kld0, kld1);
-    ld.issue_v(0, vld0, vld1);
-    ld.stage_k(k_lds[0], kld0, kld1);
-    if (nsteps > 1) ld.issue_k(1, kld0, kld1);
+    // V "of tile -1" (probabilities are zero there, but 0 * NaN is not 0)
+    const uint4 zero = make_uint4(0u, 0u, 0u, 0u);
+    uint4* v_before = v_ring + (kVStages - 1) * (kTileBytes / 16);
+    v_before[tid] = zero;
+    v_before[tid + kWaves * 64] = zero;
+    copier.issue(0, 0, 0);
+    copier.issue(1, 1, 1);
+    wait_tiles_in_flight<1>();
   }
   __syncthreads();
 
   // Tiles of this wave, in order: plain ones (every key visible to every row),
   // masked ones (the diagonal tile, or one that reaches past the last key),
-  // then tiles whose keys no row of the wave sees, where it only helps to load.
+  // then tiles whose keys no row of the wave sees, where it only helps to copy.
   // Separate loops rather than a branch inside one keep the accumulators in place.
   const int n_active = min(nsteps, wave_row0 / kKeys + 1);
   const int n_plain = min(min(wave_row0, k_end) / kKeys, n_active);
 
-  // Stage V^T of tile i and K of tile i+1 (their buffers were last read one
-  // iteration ago, before the previous barrier) and fetch the tiles after them.
-#define NVJ_STAGE_TILES(i)                                        \
-  do {                                                            \
-    ld.stage_v(vt_lds[(i) & 1], vld0, vld1);                      \
-    if ((i) + 1 < nsteps) {                                       \
-      ld.stage_k(k_lds[((i) + 1) & 1], kld0, kld1);               \
-      ld.issue_v((i) + 1, vld0, vld1);                            \
-      if ((i) + 2 < nsteps) ld.issue_k((i) + 2, kld0, kld1);      \
-    }                                                             \
+  int k_stage = 0;   // ring slot of K of tile i
+  int v_stage = 0;   // ring slot of V of tile i (tile i-1 sits one slot before)
+#define NVJ_NEXT_TILE(i)                                                              \
+  do {                                                                                \
+    copier.issue((i) + 2, k_stage >= 1 ? k_stage - 1 : kKStages - 1,                  \
+                 v_stage >= 2 ? v_stage - 2 : v_stage + kVStages - 2);                \
+    wait_tiles_in_flight<1>();                                                        \
+    __syncthreads();                                                                  \
+    k_stage = k_stage + 1 == kKStages ? 0 : k_stage + 1;                              \
+    v_stage = v_stage + 1 == kVStages ? 0 : v_stage + 1;                              \
   } while (0)
+#define NVJ_V_BEFORE() (v_lds + (v_stage >= 1 ? v_stage - 1 : kVStages - 1) * kTileBytes)
 
   f32x4 sc[2][2];
   bf16x8 pb[2];
   pb[0] = pb[1] = as_bf16x8(make_uint4(0u, 0u, 0u, 0u));
   int i = 0;
   for (; i < n_plain; ++i) {
-    scores_of_tile(k_lds[i & 1], qreg, sc, r, kg);
-    NVJ_STAGE_TILES(i);
-    accumulate_tile(vt_lds[(i & 1) ^ 1], pb, acc, lacc, r, kg);
+    scores_of_tile(k_lds + k_stage * kTileBytes, qreg, sc, r, kg);
+    accumulate_tile(NVJ_V_BEFORE(), pb, acc, lacc, r, kg);
     probabilities_of_tile<false>(sc, pb, acc, lacc, m_run, mneg, sl2, r, kg, 0, 0);
-    __syncthreads();
+    NVJ_NEXT_TILE(i);
   }
   for (; i < n_active; ++i) {
     const int ks = i * kKeys;
-    scores_of_tile(k_lds[i & 1], qreg, sc, r, kg);
-    NVJ_STAGE_TILES(i);
-    accumulate_tile(vt_lds[(i & 1) ^ 1], pb, acc, lacc, r, kg);
+    scores_of_tile(k_lds + k_stage * kTileBytes, qreg, sc, r, kg);
+    accumulate_tile(NVJ_V_BEFORE(), pb, acc, lacc, r, kg);
     probabilities_of_tile<true>(sc, pb, acc, lacc, m_run, mneg, sl2, r, kg, wave_row0 - ks,
                                 k_end - 1 - ks);
-    __syncthreads();
+    NVJ_NEXT_TILE(i);
   }
-  // the last tile of the wave is still to be accumulated; its V^T stays in
-  // place until the staging of the iteration after this one
-  if (n_active > 0) accumulate_tile(vt_lds[(n_active - 1) & 1], pb, acc, lacc, r, kg);
-  for (; i < nsteps; ++i) {
-    NVJ_STAGE_TILES(i);
-    __syncthreads();
-  }
-#undef NVJ_STAGE_TILES
+  // the last tile of the wave is still to be accumulated; its V stays in place
+  // until the copies of two iterations from now
+  if (n_active > 0) accumulate_tile(NVJ_V_BEFORE(), pb, acc, lacc, r, kg);
+  for (; i < nsteps; ++i) NVJ_NEXT_TILE(i);
+  wait_tiles_in_flight<0>();   // copies past the last tile are still landing in LDS
+#undef NVJ_NEXT_TILE
+#undef NVJ_V_BEFORE
 
-  // ---- epilogue: acc[g][jd][e] is O[row][dim = 32*kg + 8*e + jd] ----
+  // ---- epilogue: acc[g][jd][e] is O[row][dim = 16*jd + 4*kg + e] ----
 #pragma unroll
   for (int g = 0; g < 2; ++g) {
     const float l = lacc[g][0];   // already summed over every key of the row
     const int row = wave_row0 + 16 * g + r;
     if (row < len_q) {
       const float inv = l > 0.f ? 1.0f / l : 0.f;   // no visible key at all -> zeros
-      uint4* orow = a.out + ((int64_t)(q_base + row) * a.num_heads + head) * kPieces + 4 * kg;
+      uint2* orow = reinterpret_cast<uint2*>(
+          a.out + ((int64_t)(q_base + row) * a.num_heads + head) * kPieces);
 #pragma unroll
-      for (int e = 0; e < 4; ++e) {
-        uint4 o;
-        o.x = pack_bf16x2(acc[g][0][e] * inv, acc[g][1][e] * inv);
-        o.y = pack_bf16x2(acc[g][2][e] * inv, acc[g][3][e] * inv);
-        o.z = pack_bf16x2(acc[g][4][e] * inv, acc[g][5][e] * inv);
-        o.w = pack_bf16x2(acc[g][6][e] * inv, acc[g][7][e] * inv);
-        orow[e] = o;
+      for (int jd = 0; jd < 8; ++jd) {
+        uint2 o;
+        o.x = pack_bf16x2(acc[g][jd][0] * inv, acc[g][jd][1] * inv);
+        o.y = pack_bf16x2(acc[g][jd][2] * inv, acc[g][jd][3] * inv);
+        orow[4 * jd + kg] = o;
       }
     }
   }
