@@ -40,9 +40,13 @@ typedef __attribute__((ext_vector_type(4))) float f32x4;
 
 constexpr int kD = 128;
 constexpr int kPieces = 16;          // 16-byte pieces per (position, head) row
-constexpr int kBM = 128;             // query rows per workgroup
+// 2 groups x 4 waves (128 query rows, two workgroups per CU) measured fastest:
+// 4 groups x 4 waves (one wave per SIMD, accumulators in AGPRs) and 8-wave
+// workgroups (1 or 2 groups) were 5-20 % slower.
+constexpr int kGroups = 2;           // column groups of 16 query rows per wave
 constexpr int kWaves = 4;
-constexpr int kRowsPerWave = kBM / kWaves;   // 32 = two column groups of 16
+constexpr int kRowsPerWave = 16 * kGroups;
+constexpr int kBM = kRowsPerWave * kWaves;   // query rows per workgroup
 constexpr int kKeys = 32;            // keys per step
 constexpr int kTileBytes = kKeys * kD * 2;   // one K or V tile in LDS: 32 rows of 256 bytes
 constexpr int kKStages = 3;          // K tiles i .. i+2 are live in iteration i
@@ -94,11 +98,13 @@ __device__ __forceinline__ void copy16_to_lds(const char* base, uint32_t offset,
 }
 
 // Cooperative tile copies of a workgroup.  A tile is 512 pieces of K and 512 of
-// V; wave w copies rows 8w .. 8w+7 of both with two instructions each (4 rows =
-// 1024 contiguous LDS bytes per instruction).  Lane l of instruction j writes
-// position l % 16 of row 8w + 4j + l / 16 and fetches the piece that belongs
-// there.  Rows are clamped to the last visible key, so nothing at or beyond
+// V; each wave copies its share of the rows of both (8 rows with 4 waves), 4
+// rows = 1024 contiguous LDS bytes per instruction.  Lane l of instruction j of
+// wave w writes position l % 16 of row 8w + 4j + l / 16 and fetches the piece
+// that belongs there.  Rows are clamped to the last visible key, so nothing at or beyond
 // k_end is read.
+constexpr int kCopyRowsPerWave = kKeys / kWaves;   // rows of a tile one wave copies
+static_assert(kCopyRowsPerWave % 4 == 0, "one copy instruction covers 4 rows");
 struct TileCopier {
   const char* k_head;   // first key row of the sequence for this kv head
   const char* v_head;
@@ -113,10 +119,10 @@ struct TileCopier {
     const char* kb = k_head + (size_t)ks * row_bytes;
     const char* vb = v_head + (size_t)ks * row_bytes;
 #pragma unroll
-    for (int j = 0; j < 2; ++j) {
-      const int row = 8 * wave + 4 * j + (lane >> 4);
+    for (int j = 0; j < kCopyRowsPerWave / 4; ++j) {
+      const int row = kCopyRowsPerWave * wave + 4 * j + (lane >> 4);
       const uint32_t row_off = __umul24(min(row, cap), row_bytes);
-      const uint32_t dst = (uint32_t)(2 * wave + j) * 1024u;
+      const uint32_t dst = (uint32_t)(kCopyRowsPerWave / 4 * wave + j) * 1024u;
       copy16_to_lds(kb, row_off + 16u * k_position(row, lane & 15),
                     k_lds + (uint32_t)k_stage * kTileBytes + dst);
       copy16_to_lds(vb, row_off + 16u * v_position(row, lane & 15),
@@ -124,16 +130,17 @@ struct TileCopier {
     }
   }
 };
-constexpr int kCopiesPerTile = 4;   // copy16_to_lds calls of one lane per tile
+constexpr int kCopiesPerTile = 2 * (kCopyRowsPerWave / 4);   // copy16_to_lds calls of one lane per tile
 
 // Blocks until at most `tiles` of this lane's most recent tile copies are still
 // in flight (vmcnt counts the copies in order).
 template <int TILES>
 __device__ __forceinline__ void wait_tiles_in_flight() {
   static_assert(TILES == 0 || TILES == 1, "vmcnt immediates below");
+  static_assert(kCopiesPerTile == 4 || kCopiesPerTile == 2, "vmcnt immediates below");
   if (TILES == 0) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-  else asm volatile("s_waitcnt vmcnt(4)" ::: "memory");
-  static_assert(kCopiesPerTile == 4, "vmcnt immediates above");
+  else if (kCopiesPerTile == 4) asm volatile("s_waitcnt vmcnt(4)" ::: "memory");
+  else asm volatile("s_waitcnt vmcnt(2)" ::: "memory");
 }
 
 // NaN-propagating maximum: one v_maximum3_f32 per three values, no
@@ -149,8 +156,8 @@ __device__ __forceinline__ float max_of8(const f32x4& a, const f32x4& b) {
 
 // S^T of one 32-key tile against both column groups (16 query rows each):
 // sc[g][h] holds keys 16*h + 4*kg + e of the tile for query row r of group g.
-__device__ __forceinline__ void scores_of_tile(lds_ptr kt, const bf16x8 (&qreg)[2][4],
-                                               f32x4 (&sc)[2][2], int r, int kg) {
+__device__ __forceinline__ void scores_of_tile(lds_ptr kt, const bf16x8 (&qreg)[kGroups][4],
+                                               f32x4 (&sc)[kGroups][2], int r, int kg) {
   bf16x8 ka[2][4];
 #pragma unroll
   for (int s = 0; s < 4; ++s) {
@@ -160,7 +167,7 @@ __device__ __forceinline__ void scores_of_tile(lds_ptr kt, const bf16x8 (&qreg)[
     ka[1][s] = *reinterpret_cast<const __attribute__((address_space(3))) bf16x8*>(kt + at + 16 * 256);
   }
 #pragma unroll
-  for (int g = 0; g < 2; ++g) {
+  for (int g = 0; g < kGroups; ++g) {
     sc[g][0] = sc[g][1] = f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
     for (int s = 0; s < 4; ++s) {
@@ -181,8 +188,8 @@ __device__ __forceinline__ void scores_of_tile(lds_ptr kt, const bf16x8 (&qreg)[
 // Every element of lacc[g] of a lane is the sum over all 32 keys of the tile for
 // the lane's query row: a ones-row times P^T on the matrix core, from the same
 // bf16 probabilities as the numerator.
-__device__ __forceinline__ void accumulate_tile(lds_ptr vt, const bf16x8 (&pb)[2],
-                                                f32x4 (&acc)[2][8], f32x4 (&lacc)[2], int r,
+__device__ __forceinline__ void accumulate_tile(lds_ptr vt, const bf16x8 (&pb)[kGroups],
+                                                f32x4 (&acc)[kGroups][8], f32x4 (&lacc)[kGroups], int r,
                                                 int kg) {
   const int row = 4 * kg + (r >> 2);   // (16 + row) & 7 == row & 7: both reads share positions
   const int chunk = r & 3;             // 8-byte chunk of the 32 bytes of a dimension group
@@ -199,7 +206,7 @@ __device__ __forceinline__ void accumulate_tile(lds_ptr vt, const bf16x8 (&pb)[2
   const uint32_t one2 = 0x3F803F80u;   // two bf16 ones
   const bf16x8 ones = as_bf16x8(make_uint4(one2, one2, one2, one2));
 #pragma unroll
-  for (int g = 0; g < 2; ++g) {
+  for (int g = 0; g < kGroups; ++g) {
     lacc[g] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ones, pb[g], lacc[g], 0, 0, 0);
 #pragma unroll
     for (int jd = 0; jd < 8; ++jd)
@@ -215,13 +222,13 @@ __device__ __forceinline__ void accumulate_tile(lds_ptr vt, const bf16x8 (&pb)[2
 // Must run after the previous tile has been accumulated: moving the reference
 // point rescales acc and lacc.
 template <bool MASK>
-__device__ __forceinline__ void probabilities_of_tile(f32x4 (&sc)[2][2], bf16x8 (&pb)[2],
-                                                      f32x4 (&acc)[2][8], f32x4 (&lacc)[2],
-                                                      float (&m_run)[2], float (&mneg)[2],
+__device__ __forceinline__ void probabilities_of_tile(f32x4 (&sc)[kGroups][2], bf16x8 (&pb)[kGroups],
+                                                      f32x4 (&acc)[kGroups][8], f32x4 (&lacc)[kGroups],
+                                                      float (&m_run)[kGroups], float (&mneg)[kGroups],
                                                       float sl2, int r, int kg, int row_limit,
                                                       int key_limit) {
 #pragma unroll
-  for (int g = 0; g < 2; ++g) {
+  for (int g = 0; g < kGroups; ++g) {
     f32x4& s0 = sc[g][0];
     f32x4& s1 = sc[g][1];
     // lane = (query row r of the group, key group kg): keys 4*kg + e and
@@ -288,7 +295,7 @@ struct PrefillArgs {
 };
 
 // grid.x = 8 * ceil(tile bound * Hq / 8) workgroups (see the work-item mapping below).
-__global__ __launch_bounds__(kWaves * 64, 2) void prefill_attention_kernel(PrefillArgs a,
+__global__ __launch_bounds__(kWaves * 64, kGroups <= 2 ? 2 : 1) void prefill_attention_kernel(PrefillArgs a,
                                                                         int num_tiles_bound) {
   __shared__ uint4 k_ring[kKStages * kTileBytes / 16];
   __shared__ uint4 v_ring[kVStages * kTileBytes / 16];
@@ -341,9 +348,9 @@ __global__ __launch_bounds__(kWaves * 64, 2) void prefill_attention_kernel(Prefi
 
   // ---- Q^T of both column groups as B operands: column r of group g is row
   // q0 + 32*wave + 16*g + r; rows beyond the sequence are zero ----
-  bf16x8 qreg[2][4];
+  bf16x8 qreg[kGroups][4];
 #pragma unroll
-  for (int g = 0; g < 2; ++g) {
+  for (int g = 0; g < kGroups; ++g) {
     const int row = q0 + kRowsPerWave * wave + 16 * g + r;
     const uint4 zero = make_uint4(0u, 0u, 0u, 0u);
     const uint4* qrow =
@@ -367,10 +374,10 @@ __global__ __launch_bounds__(kWaves * 64, 2) void prefill_attention_kernel(Prefi
                              (uint32_t)(uintptr_t)v_lds, k_end - 1, nsteps - 1, wave, lane};
 
   const float sl2 = a.scale_log2e;
-  f32x4 acc[2][8], lacc[2];
-  float m_run[2], mneg[2];
+  f32x4 acc[kGroups][8], lacc[kGroups];
+  float m_run[kGroups], mneg[kGroups];
 #pragma unroll
-  for (int g = 0; g < 2; ++g) {
+  for (int g = 0; g < kGroups; ++g) {
     m_run[g] = kNegBig;
     mneg[g] = -kNegBig * sl2;
     lacc[g] = f32x4{0.f, 0.f, 0.f, 0.f};
@@ -390,8 +397,7 @@ __global__ __launch_bounds__(kWaves * 64, 2) void prefill_attention_kernel(Prefi
     // V "of tile -1" (probabilities are zero there, but 0 * NaN is not 0)
     const uint4 zero = make_uint4(0u, 0u, 0u, 0u);
     uint4* v_before = v_ring + (kVStages - 1) * (kTileBytes / 16);
-    v_before[tid] = zero;
-    v_before[tid + kWaves * 64] = zero;
+    for (int p = tid; p < kTileBytes / 16; p += kWaves * 64) v_before[p] = zero;
     copier.issue(0, 0, 0);
     copier.issue(1, 1, 1);
     wait_tiles_in_flight<1>();
@@ -402,7 +408,7 @@ __global__ __launch_bounds__(kWaves * 64, 2) void prefill_attention_kernel(Prefi
   // masked ones (the diagonal tile, or one that reaches past the last key),
   // then tiles whose keys no row of the wave sees, where it only helps to copy.
   // Separate loops rather than a branch inside one keep the accumulators in place.
-  const int n_active = min(nsteps, wave_row0 / kKeys + 1);
+  const int n_active = min(nsteps, (wave_row0 + kRowsPerWave - 1) / kKeys + 1);
   const int n_plain = min(min(wave_row0, k_end) / kKeys, n_active);
 
   int k_stage = 0;   // ring slot of K of tile i
@@ -418,9 +424,10 @@ __global__ __launch_bounds__(kWaves * 64, 2) void prefill_attention_kernel(Prefi
   } while (0)
 #define NVJ_V_BEFORE() (v_lds + (v_stage >= 1 ? v_stage - 1 : kVStages - 1) * kTileBytes)
 
-  f32x4 sc[2][2];
-  bf16x8 pb[2];
-  pb[0] = pb[1] = as_bf16x8(make_uint4(0u, 0u, 0u, 0u));
+  f32x4 sc[kGroups][2];
+  bf16x8 pb[kGroups];
+#pragma unroll
+  for (int g = 0; g < kGroups; ++g) pb[g] = as_bf16x8(make_uint4(0u, 0u, 0u, 0u));
   int i = 0;
   for (; i < n_plain; ++i) {
     scores_of_tile(k_lds + k_stage * kTileBytes, qreg, sc, r, kg);
@@ -446,7 +453,7 @@ __global__ __launch_bounds__(kWaves * 64, 2) void prefill_attention_kernel(Prefi
 
   // ---- epilogue: acc[g][jd][e] is O[row][dim = 16*jd + 4*kg + e] ----
 #pragma unroll
-  for (int g = 0; g < 2; ++g) {
+  for (int g = 0; g < kGroups; ++g) {
     const float l = lacc[g][0];   // already summed over every key of the row
     const int row = wave_row0 + 16 * g + r;
     if (row < len_q) {
