@@ -252,6 +252,44 @@ NVJ_API int nvj_prefill_attention_launch(void* stream, const void* q, const void
                             int32_t total_q_tokens, int32_t batch, int32_t num_heads,
                             int32_t num_kv_heads, int32_t head_dim, float scale);
 
+/*
+ * RMSNorm over the last dimension, optionally fused with the residual add.
+ * Replaces RMSNorm._rms_forward (layers/layernorm.py:31-48) when `residual` is
+ * NULL and RMSNorm._add_rms_forward (layers/layernorm.py:50-79) otherwise, as
+ * called around every attention and MLP block (models/qwen3.py:305-313, 364).
+ *
+ *   x            [num_tokens, hidden] bf16
+ *   residual     [num_tokens, hidden] bf16 or NULL
+ *   weight       [hidden] float32
+ *   y            [num_tokens, hidden] bf16: bf16((s * rsqrt(mean(s^2) + eps)) * weight)
+ *   residual_out [num_tokens, hidden] bf16: bf16(s); NULL exactly when residual is
+ *
+ * with s = float(x) + float(residual) (or float(x)); the mean is taken over the
+ * unrounded fp32 sums, as the reference does.  residual_out may be the same
+ * buffer as residual; x and y must not overlap any other argument.  hidden must
+ * be a multiple of 8 and at most 8192; all pointers 16-byte aligned.
+ */
+NVJ_API int nvj_add_rms_norm_launch(void* stream, const void* x, const void* residual,
+                            const float* weight, float eps, void* y, void* residual_out,
+                            int32_t num_tokens, int32_t hidden);
+
+/*
+ * SiLU(gate) * up for the fused gate/up projection of the MLP.  Replaces
+ * SiluAndMul.__call__ (layers/activation.py:22-33; called at
+ * models/qwen3.py:229).
+ *
+ *   x [num_tokens, x_row_stride] bf16: gate in columns [0, intermediate), up in
+ *     [intermediate, 2 * intermediate) of every row (x_row_stride >= 2 *
+ *     intermediate elements, a multiple of 8)
+ *   y [num_tokens, intermediate] bf16
+ *
+ * Evaluated in fp32 from the bf16 inputs and rounded once to bf16 (the reference
+ * leaves the rounding points of the bf16 expression to XLA).  intermediate must
+ * be a multiple of 8; pointers 16-byte aligned.
+ */
+NVJ_API int nvj_silu_and_mul_launch(void* stream, const void* x, int64_t x_row_stride,
+                            void* y, int32_t num_tokens, int32_t intermediate);
+
 #ifdef __cplusplus
 }  /* extern "C" */
 #endif

@@ -47,6 +47,11 @@ SYMBOLS = {
     "nvj_prefill_attention_launch": (_c.c_int, [
         _c.c_void_p, _c.c_void_p, _c.c_void_p, _c.c_void_p, _c.c_void_p, _c.c_void_p, _c.c_void_p,
         _c.c_int32, _c.c_int32, _c.c_int32, _c.c_int32, _c.c_int32, _c.c_float]),
+    "nvj_add_rms_norm_launch": (_c.c_int, [
+        _c.c_void_p, _c.c_void_p, _c.c_void_p, _c.c_void_p, _c.c_float, _c.c_void_p, _c.c_void_p,
+        _c.c_int32, _c.c_int32]),
+    "nvj_silu_and_mul_launch": (_c.c_int, [
+        _c.c_void_p, _c.c_void_p, _c.c_int64, _c.c_void_p, _c.c_int32, _c.c_int32]),
 }
 NVJ_PHASE_SPLITK = 1
 NVJ_PHASE_COMBINE = 2

@@ -19,7 +19,7 @@ LIB_NAME = "libnvj_paged_attn.so"
 LIB_PATH = os.path.join(NATIVE_DIR, LIB_NAME)
 
 SOURCES = ("store_kvcache.hip", "paged_decode.hip", "qk_norm_rope_store.hip",
-           "decode_metadata.hip", "prefill_attention.hip")
+           "decode_metadata.hip", "prefill_attention.hip", "layer_glue.hip")
 
 HIPCC_FLAGS = (
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-shared",

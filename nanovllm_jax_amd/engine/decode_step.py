@@ -1,9 +1,11 @@
 """Whole-model decode step harness around the HIP attention path.
 
 The measured path of this package is the KV-cache store and the paged decode
-attention; everything else a decode step needs (embedding, RMSNorm, the QKV /
-output / MLP projections, RoPE, the LM head, greedy pick) is plain
-``torch`` here (hipBLASLt GEMMs), written from the architecture the reference
+attention, with the element-wise stages next to it (QK-RMSNorm + RoPE + store,
+RMSNorm + residual, SiLU-and-multiply) as single HIP launches; the rest of a
+decode step (embedding, the QKV / output / MLP projections, the LM head,
+greedy pick) is plain ``torch`` here (hipBLASLt GEMMs), written from the
+architecture the reference
 describes: ``models/qwen3.py:130-172`` (attention block: fused QKV, per-head
 QK-RMSNorm when there is no QKV bias, RoPE, attention, output projection),
 ``:285-318`` (pre-norm decoder layer with fused residual), ``:366-393`` (stack
@@ -25,7 +27,9 @@ import torch
 import torch.nn.functional as F
 
 from .. import _lib
+from ..layers.activation import silu_and_mul
 from ..layers.attention import Attention
+from ..layers.layernorm import rms_norm
 from ..layers.paged_attention import paged_attention, paged_decode_workspace_bytes
 from ..layers.prefill_attention import variable_length_attention_prefill
 from ..layers.qk_rope_store import qk_norm_rope_store
@@ -141,8 +145,12 @@ class DecodeStepRunner:
     ``Attention`` per layer; ``step`` runs one decode step for a batch."""
 
     def __init__(self, cfg: DecodeModelConfig, device="cuda:0", seed: int = 0,
-                 fill_cache: bool = True, fused_qk_rope_store: bool = True):
+                 fill_cache: bool = True, fused_qk_rope_store: bool = True,
+                 fused_layer_glue: bool = True):
         self.cfg = cfg
+        # True: RMSNorm (+ residual add) and SiLU-and-multiply as one HIP launch
+        # each; False: the same stages as chains of torch kernels
+        self.fused_layer_glue = fused_layer_glue
         # True: one HIP launch for QK-RMSNorm + RoPE + KV store; False: the
         # reference's op-by-op chain in torch followed by the plain store
         self.fused_qk_rope_store = fused_qk_rope_store
@@ -160,15 +168,15 @@ class DecodeStepRunner:
         self.layers = []
         for _ in range(c.num_layers):
             self.layers.append(dict(
-                ln1=torch.ones(c.hidden_size, device=self.device, dtype=torch.bfloat16),
-                ln2=torch.ones(c.hidden_size, device=self.device, dtype=torch.bfloat16),
+                ln1=torch.ones(c.hidden_size, device=self.device),    # fp32, layernorm.py:29
+                ln2=torch.ones(c.hidden_size, device=self.device),
                 qkv=w(qkv_out, c.hidden_size),
                 o=w(c.hidden_size, c.num_heads * c.head_dim),
                 q_norm=torch.ones(c.head_dim, device=self.device),
                 k_norm=torch.ones(c.head_dim, device=self.device),
                 gate_up=w(2 * c.intermediate_size, c.hidden_size),
                 down=w(c.hidden_size, c.intermediate_size)))
-        self.final_norm = torch.ones(c.hidden_size, device=self.device, dtype=torch.bfloat16)
+        self.final_norm = torch.ones(c.hidden_size, device=self.device)
         inv_freq = 1.0 / (c.rope_theta ** (torch.arange(0, c.head_dim, 2, dtype=torch.float32,
                                                         device=self.device) / c.head_dim))
         freqs = torch.outer(torch.arange(c.max_position, dtype=torch.float32,
@@ -193,13 +201,24 @@ class DecodeStepRunner:
 
     # -- small torch pieces -------------------------------------------------
     def _rms(self, x, weight, residual=None):
-        """RMSNorm, optionally fused with the residual add (layernorm.py:31-79):
-        the sum is taken in fp32 and rounded once to the model dtype, which is
-        both the new residual and the input of the norm (the reference norms
-        the unrounded fp32 sum; the difference is one bf16 rounding)."""
+        """RMSNorm, optionally fused with the residual add (layernorm.py:31-79).
+        The HIP launch norms the unrounded fp32 sum as the reference does and
+        updates the residual in place; the torch chain rounds the sum to the
+        model dtype first (one bf16 rounding apart)."""
+        if self.fused_layer_glue and x.dim() == 2:
+            if residual is None:
+                return rms_norm(x, weight, self.cfg.rms_norm_eps), x
+            return rms_norm(x, weight, self.cfg.rms_norm_eps, residual, residual_out=residual)
         if residual is not None:
             x = (x.float() + residual.float()).to(x.dtype)
         return F.rms_norm(x, (x.shape[-1],), weight.to(x.dtype), self.cfg.rms_norm_eps), x
+
+    def _silu_mul(self, gate_up):
+        """SiLU(gate) * up of the fused projection (activation.py:22-33)."""
+        if self.fused_layer_glue:
+            return silu_and_mul(gate_up)
+        gate, up = gate_up.chunk(2, dim=-1)
+        return F.silu(gate) * up
 
     def _rope(self, x, cos, sin):
         """x bf16 [T, H, D]; result float32 like the reference's promotion
@@ -240,8 +259,7 @@ class DecodeStepRunner:
                                         workspace=attn.workspace)
                 h = F.linear(o.reshape(-1, qs), lw["o"])
                 h, residual = self._rms(h, lw["ln2"], residual)
-                gate, up = F.linear(h, lw["gate_up"]).chunk(2, dim=-1)
-                h = F.linear(F.silu(gate) * up, lw["down"])
+                h = F.linear(self._silu_mul(F.linear(h, lw["gate_up"])), lw["down"])
                 continue
             q, k, v = qkv.split([qs, ks, ks], dim=-1)
             q = q.reshape(-1, c.num_heads, c.head_dim)
@@ -254,8 +272,7 @@ class DecodeStepRunner:
             o = attn(q.to(torch.bfloat16).contiguous(), k, v, context)
             h = F.linear(o.reshape(-1, qs), lw["o"])
             h, residual = self._rms(h, lw["ln2"], residual)
-            gate, up = F.linear(h, lw["gate_up"]).chunk(2, dim=-1)
-            h = F.linear(F.silu(gate) * up, lw["down"])
+            h = F.linear(self._silu_mul(F.linear(h, lw["gate_up"])), lw["down"])
         h, _ = self._rms(h, self.final_norm, residual)
         if context.is_prefill:                           # only the last token of each prompt
             h = h[context.last_token_indices.long()]     # (models/qwen3.py:472-491)

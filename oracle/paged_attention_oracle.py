@@ -37,6 +37,21 @@ What pins each function (see tests/test_oracle_pinning.py):
                                   first V row; packing invariance (a batch equals
                                   its sequences run one by one).  Same unpinned
                                   bf16 rounding of probabilities as the fallback.
+* ``add_rms_norm_ref``          - float64 RMSNorm of the float64 sum (closed form),
+                                  ``torch.nn.functional.rms_norm`` in float32; unit
+                                  weight gives unit RMS; the residual output is
+                                  the bf16 rounding of the exact sum.  The fp32
+                                  summation order of the mean is this oracle's
+                                  choice (the reference leaves it to XLA): PARITY
+                                  UNPINNED at the level of fp32 round-off of that
+                                  sum.
+* ``silu_and_mul_ref``          - float64 ``g / (1 + exp(-g)) * u`` and torch's
+                                  ``silu`` in float64; silu(0) = 0, large gates
+                                  pass ``up`` through, large negative gates give 0.
+                                  Evaluated in float64 and rounded once to bf16;
+                                  where XLA rounds inside the reference's bf16
+                                  expression is PARITY UNPINNED (at most one bf16
+                                  ulp per rounding point).
 * ``paged_attention_fallback_ref``
                                 - same checks; the bf16 rounding of the
                                   probabilities inside ``jax.nn.dot_product_attention``
@@ -67,6 +82,8 @@ __all__ = [
     "textbook_prefill_f64",
     "prepare_decode_ref",
     "advance_decode_ref",
+    "add_rms_norm_ref",
+    "silu_and_mul_ref",
 ]
 
 
@@ -530,3 +547,59 @@ def textbook_prefill_f64(q, k, v, cu_seqlens_q, cu_seqlens_k, scale):
                 w /= w.sum()
                 out[q0 + row, h] = sum(w[j] * vf[k0 + j, h // G] for j in range(n))
     return out
+
+
+# ---------------------------------------------------------------------------
+# RMSNorm (+ residual) and SiLU-and-multiply
+# ---------------------------------------------------------------------------
+def add_rms_norm_ref(x, weight, eps, residual=None):
+    """``RMSNorm._rms_forward`` / ``_add_rms_forward`` (layers/layernorm.py:31-79).
+
+    ``x``, ``residual``: ``[T, hidden]`` bf16 bit patterns (uint16); ``weight``
+    ``[hidden]`` float32.  Returns ``y`` bits, or ``(y, new_residual)`` bits.
+
+    fp32 throughout as the reference (:41, :66); the order of the sum of squares
+    is this oracle's choice: the row is cut into 8-element pieces, accumulator
+    ``l`` (of 64) takes pieces ``l, l + 64, ...`` in row order, then the 64
+    accumulators are folded pairwise at distances 32, 16, ..., 1.
+    """
+    xb = _as_bf16_bits(np.asarray(x))
+    t, hidden = xb.shape
+    assert hidden % 8 == 0
+    s = bf16_bits_to_f32(xb)
+    new_res = None
+    if residual is not None:
+        s = (s + bf16_bits_to_f32(_as_bf16_bits(np.asarray(residual)))).astype(np.float32)
+        new_res = f32_to_bf16_bits(s)                          # :68-69
+    pieces = hidden // 8
+    sq = (s * s).astype(np.float32).reshape(t, pieces, 8)
+    acc = np.zeros((t, 64), np.float32)
+    for p in range(pieces):
+        lane = p % 64
+        for e in range(8):
+            acc[:, lane] = (acc[:, lane] + sq[:, p, e]).astype(np.float32)
+    m = 32
+    while m >= 1:
+        idx = np.arange(64) ^ m
+        acc = (acc + acc[:, idx]).astype(np.float32)
+        m >>= 1
+    total = acc[:, :1]
+    inv_hidden = np.float32(1.0) / np.float32(hidden)
+    r = (np.float32(1.0) / np.sqrt((total * inv_hidden + np.float32(eps)).astype(np.float32))
+         ).astype(np.float32)                                  # :72-73
+    w = np.asarray(weight, np.float32)[None, :]
+    y = f32_to_bf16_bits(((s * r).astype(np.float32) * w).astype(np.float32))   # :76
+    return y if residual is None else (y, new_res)
+
+
+def silu_and_mul_ref(x):
+    """``SiluAndMul.__call__`` (layers/activation.py:22-33): ``x`` ``[T, 2*I]`` bf16
+    bits -> ``[T, I]`` bf16 bits, ``silu(gate) * up`` evaluated in float64 from the
+    bf16 inputs and rounded once (via float32) to bf16."""
+    xb = _as_bf16_bits(np.asarray(x))
+    inter = xb.shape[-1] // 2
+    g = bf16_bits_to_f32(xb[..., :inter]).astype(np.float64)
+    u = bf16_bits_to_f32(xb[..., inter:]).astype(np.float64)
+    with np.errstate(over="ignore"):
+        out = g / (1.0 + np.exp(-g)) * u
+    return f32_to_bf16_bits(out.astype(np.float32))

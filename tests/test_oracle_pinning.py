@@ -385,3 +385,58 @@ def test_prefill_against_torch_sdpa_causal_gqa_and_packing_invariance():
         alone = variable_length_attention_prefill_ref(q[sl], k[sl], v[sl], [0, n], [0, n],
                                                       D ** -0.5, return_f32=True)
         assert np.array_equal(alone, got[sl])
+
+
+# ---------------------------------------------------------------------------
+# RMSNorm (+ residual) and SiLU-and-multiply
+# ---------------------------------------------------------------------------
+@pytest.mark.parametrize("hidden", [1024, 520, 4096])
+def test_add_rms_norm_against_float64_and_torch(hidden):
+    import torch
+    from oracle.paged_attention_oracle import add_rms_norm_ref
+    rng = np.random.Generator(np.random.PCG64(61))
+    x = f32_to_bf16_bits(rng.standard_normal((5, hidden), dtype=np.float32) * 3)
+    res = f32_to_bf16_bits(rng.standard_normal((5, hidden), dtype=np.float32))
+    w = (1 + 0.3 * rng.standard_normal(hidden)).astype(np.float32)
+    xf, rf = bf16_bits_to_f32(x).astype(np.float64), bf16_bits_to_f32(res).astype(np.float64)
+
+    # closed form in float64 (layers/layernorm.py:41-48 and :66-76)
+    def f64(s):
+        return s / np.sqrt((s * s).mean(-1, keepdims=True) + 1e-6) * w
+
+    y = bf16_bits_to_f32(add_rms_norm_ref(x, w, 1e-6))
+    want = f64(xf)
+    assert np.all(np.abs(y - want) <= 2.0 ** -8 * np.abs(want) + 1e-30)       # one bf16 rounding
+    y2, new_res = add_rms_norm_ref(x, w, 1e-6, res)
+    want2 = f64(xf + rf)
+    assert np.all(np.abs(bf16_bits_to_f32(y2) - want2) <= 2.0 ** -8 * np.abs(want2) + 1e-30)
+    # the new residual is the rounding of the exact sum (a sum of two bf16 fits fp32 exactly
+    # unless the exponents are far apart, where fp32 rounds first: compare through fp32)
+    assert np.array_equal(new_res, f32_to_bf16_bits((xf + rf).astype(np.float32)))
+    # library special case: torch's rms_norm in float32
+    t = torch.nn.functional.rms_norm(torch.from_numpy(xf.astype(np.float32)), (hidden,),
+                                     torch.from_numpy(w), 1e-6).numpy()
+    assert np.all(np.abs(y - t) <= 2.0 ** -8 * np.abs(t) + 1e-30)
+    # unit weight -> unit RMS (to bf16 precision)
+    y1 = bf16_bits_to_f32(add_rms_norm_ref(x, np.ones(hidden, np.float32), 1e-6))
+    assert np.allclose(np.sqrt((y1.astype(np.float64) ** 2).mean(-1)), 1.0, atol=3e-3)
+
+
+def test_silu_and_mul_against_float64_torch_and_closed_forms():
+    import torch
+    from oracle.paged_attention_oracle import silu_and_mul_ref
+    rng = np.random.Generator(np.random.PCG64(62))
+    x = f32_to_bf16_bits(rng.standard_normal((4, 2 * 96), dtype=np.float32) * 4)
+    g = torch.from_numpy(bf16_bits_to_f32(x[:, :96]).astype(np.float64))
+    u = torch.from_numpy(bf16_bits_to_f32(x[:, 96:]).astype(np.float64))
+    want = (torch.nn.functional.silu(g) * u).numpy()
+    got = bf16_bits_to_f32(silu_and_mul_ref(x))
+    assert np.all(np.abs(got - want) <= 2.0 ** -8 * np.abs(want) + 1e-30)
+    # closed forms: silu(0) = 0; a large gate passes `up` through; a large negative gate gives 0
+    special = f32_to_bf16_bits(np.array([[0.0, 80.0, -200.0, 1.0, 1.5, -2.5, 3.0, 7.0]],
+                                          np.float32))
+    out = bf16_bits_to_f32(silu_and_mul_ref(special))
+    assert out[0, 0] == 0.0
+    assert out[0, 1] == np.float32(80.0 * -2.5)
+    assert out[0, 2] == 0.0
+    assert abs(out[0, 3] - 7.0 / (1 + np.exp(-1.0))) <= 2.0 ** -8 * 7
