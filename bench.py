@@ -28,11 +28,12 @@ if ROOT not in sys.path:
 
 HBM_PEAK_GBPS = 8000.0
 
-# HBM bytes per split-K launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of
+# HBM bytes per decode launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of
 # this very command, scaled by the same counters over a plain 1 GiB copy
 # (FETCH_SIZE x1.9999, WRITE_SIZE x1.0).  Keyed by (workload, chunk); other
 # configurations report null.
-MEASURED_TRAFFIC_BYTES = {("C2", 0): 1_080_210_000, ("C2", 1024): 1_080_188_000}
+MEASURED_TRAFFIC_BYTES = {("C2", 0): 1_080_210_000, ("C2", 1024): 1_080_188_000,
+                          ("C2", -1): 1_074_909_000}
 
 
 def device_inputs(w, torch, dev):
@@ -206,8 +207,10 @@ def main():
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--workload", default="C2", choices=["C1", "C2", "C3", "C4", "C5"])
-    ap.add_argument("--chunk", type=int, default=0,
-                    help="positions per workgroup (0 = balanced split, the default)")
+    ap.add_argument("--chunk", type=int, default=None,
+                    help="split mode: 0 = balanced, > 0 = positions per workgroup, -1 = whole "
+                         "sequence per workgroup; default: what the host filler would pick from "
+                         "the workload's lengths (layers.paged_attention.choose_split)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run a plain 1 GiB device-to-device copy a few times, so a "
@@ -233,7 +236,8 @@ def main():
               file=sys.stderr)
         return 1
     from nanovllm_jax_amd import _lib, paged_attention, store_kv_to_cache
-    from nanovllm_jax_amd.layers.paged_attention import paged_decode_workspace_bytes
+    from nanovllm_jax_amd.layers.paged_attention import (choose_split,
+                                                         paged_decode_workspace_bytes)
     from nanovllm_jax_amd.workloads import algorithmic_bytes, make_workload
 
     dev = torch.device("cuda:0")
@@ -244,7 +248,12 @@ def main():
         return bench_prefill(args, torch)
     w = make_workload(args.workload)
     q, kc, vc, bt, ctx, slots, k_new, v_new = device_inputs(w, torch, dev)
-    chunk = args.chunk
+    # like the reference's filler, the workload generator knows the lengths on the host
+    chunk = choose_split(w.context_lens, w.num_kv_heads) if args.chunk is None else args.chunk
+    split_name = {0: "balanced", -1: "whole sequence per workgroup"}.get(chunk,
+                                                                        f"fixed chunk {chunk}")
+    kernel_name = {0: "paged_decode_balanced_kernel", -1: "paged_decode_whole_kernel"}.get(
+        chunk, "paged_decode_splitk_kernel")
     ws = torch.empty(paged_decode_workspace_bytes(w.batch, w.num_heads, w.head_dim, w.max_blocks,
                                                   w.block_size, w.num_kv_heads, chunk),
                      dtype=torch.uint8, device=dev)
@@ -291,16 +300,17 @@ def main():
                                f"D={w.head_dim} page={w.block_size} "
                                f"ctx={int(w.context_lens.min())}..{int(w.context_lens.max())} "
                                f"pool={w.num_blocks} pages",
-                   "split": "balanced" if chunk == 0 else f"fixed chunk {chunk}",
+                   "split": split_name,
                    "algorithmic_bytes_per_call": byts,
-                   "step": "split-K launch + combine launch"},
+                   "step": "one launch" if chunk == -1 else "split-K launch + combine launch"},
         "roofline": {"bound": "hbm", "achieved": round(gbps_kernel, 1), "peak": HBM_PEAK_GBPS,
                      "unit": "GB/s", "frac": round(gbps_kernel / HBM_PEAK_GBPS, 4),
-                     "traffic": MEASURED_TRAFFIC_BYTES.get((w.name, chunk)), "kernel": "paged_decode_balanced_kernel" if chunk == 0 else "paged_decode_splitk_kernel",
+                     "traffic": MEASURED_TRAFFIC_BYTES.get((w.name, chunk)), "kernel": kernel_name,
                      "kernel_us": round(ms_splitk * 1e3, 2)},
         # back-to-back launches of these two short kernels are paced by the host
         # (one Python -> ctypes call each), not by the kernels themselves
-        "host_paced_launch_us": {"paged_decode_combine_kernel": round(ms_combine * 1e3, 2),
+        "host_paced_launch_us": {"paged_decode_combine_kernel":
+                                 None if chunk == -1 else round(ms_combine * 1e3, 2),
                                  "store_kvcache_kernel": round(ms_store * 1e3, 2)},
     }
     if not args.no_cpu_baseline:

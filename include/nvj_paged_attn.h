@@ -35,6 +35,8 @@ extern "C" {
 #define NVJ_ERR_BAD_DTYPE     -6   /* unknown element type code                     */
 
 /* element type codes for the new K/V rows handed to the store */
+#define NVJ_CHUNK_WHOLE_SEQUENCE (-1)   /* see the split modes of the paged decode */
+
 #define NVJ_DTYPE_BF16 0
 #define NVJ_DTYPE_F32  1
 
@@ -83,6 +85,16 @@ NVJ_API int nvj_store_kvcache_launch(void* stream,
  *   chunk  > 0  fixed split: workgroup (b, c) takes positions
  *               [c * chunk, (c + 1) * chunk) of sequence b; chunk must be a
  *               multiple of 32.
+ *   chunk == NVJ_CHUNK_WHOLE_SEQUENCE (-1)
+ *               every sequence is finished inside one workgroup: a workgroup
+ *               owns 1, 2, 4 or 8 KV heads of one sequence (as many as still
+ *               give 256 workgroups) and its 8 waves split the sequence's
+ *               positions between them, merging through LDS.  No workspace, no
+ *               second pass.  For the caller that knows (as the reference's
+ *               host filler does, engine/model_runner.py:334-376) that the
+ *               sequences of the batch have similar lengths and that
+ *               batch * num_kv_heads is large enough to fill the GPU; a ragged
+ *               batch is better served by chunk == 0.
  *
  * nvj_paged_decode_default_chunk: the fixed chunk the library recommends for a
  * problem of this shape when a fixed split is wanted (a multiple of 32).
@@ -94,7 +106,8 @@ NVJ_API int32_t nvj_paged_decode_default_chunk(int32_t batch, int32_t num_kv_hea
  * Bytes of device workspace nvj_paged_decode_launch needs for the partials
  * (fp32 accumulators plus running max and sum per partial; in balanced mode
  * also batch + 1 int32 prefix sums) for the given `chunk` mode.  Returns 0 on
- * invalid arguments.
+ * invalid arguments, and for chunk == NVJ_CHUNK_WHOLE_SEQUENCE, which needs none
+ * (workspace may then be NULL).
  */
 NVJ_API size_t nvj_paged_decode_workspace_bytes(int32_t batch, int32_t num_heads,
                                         int32_t head_dim, int32_t max_blocks,
@@ -127,10 +140,11 @@ NVJ_API size_t nvj_paged_decode_workspace_bytes(int32_t batch, int32_t num_heads
  * rather than faulting.
  *
  * Two launches on `stream`: the split-K kernel (each workgroup streams its
- * share of positions for all KV heads) and the combine pass.
+ * share of positions for all KV heads) and the combine pass; one launch for
+ * chunk == NVJ_CHUNK_WHOLE_SEQUENCE.
  * Supported: head_dim 128 (every Qwen3 size) or 64 (the reference's toy test
  * shapes), num_heads / num_kv_heads <= 16, block_size a multiple of 32, chunk
- * a multiple of 32 (0 = balanced split).
+ * a multiple of 32 (0 = balanced split) or NVJ_CHUNK_WHOLE_SEQUENCE.
  */
 NVJ_API int nvj_paged_decode_launch(void* stream,
                             const void* q, const void* k_cache, const void* v_cache,

@@ -53,6 +53,7 @@ SYMBOLS = {
     "nvj_silu_and_mul_launch": (_c.c_int, [
         _c.c_void_p, _c.c_void_p, _c.c_int64, _c.c_void_p, _c.c_int32, _c.c_int32]),
 }
+NVJ_CHUNK_WHOLE_SEQUENCE = -1
 NVJ_PHASE_SPLITK = 1
 NVJ_PHASE_COMBINE = 2
 

@@ -153,13 +153,15 @@ struct DecodeArgs {
 };
 
 // One wave's share of one segment: positions [t0, t1) of sequence b for KV head
-// kvh.  `direct` means the segment is the whole sequence: the normalised bf16
-// result goes straight to `out`; otherwise the unnormalised partial goes to
-// partial slot `slot` of the workspace.  t0 is a multiple of 32, t0 < t1.
+// kvh; t0 is a multiple of 32, t0 < t1.  Leaves the unnormalised result in
+// registers: acc[jd][e] is O[head kvh*group + r][dim 32*kg + 8*e + jd] for the
+// lane (r = lane & 15, kg = lane >> 4), m_run the maximum raw score and l_run
+// the sum of exp((score - m_run) * scale) of that head (the same in the four
+// lanes that share r).  Lanes with r >= group hold padding.
 template <int D>
-__device__ __forceinline__ void run_segment(const DecodeArgs& a, uint4* lds, int b, int kvh,
-                                            int t0, int t1, int64_t slot, bool direct,
-                                            int lane) {
+__device__ __forceinline__ void compute_segment(const DecodeArgs& a, uint4* lds, int b, int kvh,
+                                                int t0, int t1, int lane, f32x4 (&acc)[8],
+                                                float& m_run, float& l_run) {
   using H = HeadDim<D>;
   const int r = lane & 15;   // MFMA row/column index inside a 16-wide tile
   const int kg = lane >> 4;  // MFMA k-group (which 8 of the 32 reduction slots)
@@ -208,11 +210,10 @@ __device__ __forceinline__ void run_segment(const DecodeArgs& a, uint4* lds, int
     issue_v_loads<true, D>(vreg, v_cache + off, kg, r, last, row_bytes);
   }
 
-  f32x4 acc[8];
 #pragma unroll
   for (int jd = 0; jd < 8; ++jd) acc[jd] = f32x4{0.f, 0.f, 0.f, 0.f};
-  float m_run = kNegBig;  // running max of raw scores (q.k, unscaled) of column r
-  float l_run = 0.f;      // this lane's share of the running sum
+  m_run = kNegBig;  // running max of raw scores (q.k, unscaled) of column r
+  l_run = 0.f;      // this lane's share of the running sum
 
   for (int step = 0; step < nsteps; ++step) {
     const int nvalid = min(kStep, t1 - (t0 + step * kStep));
@@ -314,34 +315,57 @@ __device__ __forceinline__ void run_segment(const DecodeArgs& a, uint4* lds, int
   // total of the running sum over the 4 k-groups that share column r
   l_run += __shfl_xor(l_run, 16, 64);
   l_run += __shfl_xor(l_run, 32, 64);
+}
 
-  if (r >= group) return;
-  const int head = kvh * group + r;
-  // acc[jd][e] is O[head][dim = 32*kg + 8*e + jd]; at head_dim 64 only k-groups
-  // 0 and 1 hold real dims
-  if (32 * kg >= D) return;
-  if (direct) {
-    const float inv = 1.0f / (l_run + 1e-9f);
-    uint4* orow = a.out + ((int64_t)b * num_heads + head) * H::kPieces + 4 * kg;
+// Normalised bf16 result of a whole sequence straight to `out`.
+template <int D>
+__device__ __forceinline__ void write_output(const DecodeArgs& a, int b, int kvh, int lane,
+                                             const f32x4 (&acc)[8], float l_run) {
+  using H = HeadDim<D>;
+  const int r = lane & 15, kg = lane >> 4;
+  // at head_dim 64 only k-groups 0 and 1 hold real dims
+  if (r >= a.group || 32 * kg >= D) return;
+  const int head = kvh * a.group + r;
+  const float inv = 1.0f / (l_run + 1e-9f);
+  uint4* orow = a.out + ((int64_t)b * a.num_heads + head) * H::kPieces + 4 * kg;
 #pragma unroll
-    for (int e = 0; e < 4; ++e) {
-      uint4 o;
-      o.x = pack_bf16x2(acc[0][e] * inv, acc[1][e] * inv);
-      o.y = pack_bf16x2(acc[2][e] * inv, acc[3][e] * inv);
-      o.z = pack_bf16x2(acc[4][e] * inv, acc[5][e] * inv);
-      o.w = pack_bf16x2(acc[6][e] * inv, acc[7][e] * inv);
-      orow[e] = o;
-    }
-  } else {
-    const int64_t row = slot * num_heads + head;
-    float4* prow = reinterpret_cast<float4*>(a.part_o + row * D + 32 * kg);
-#pragma unroll
-    for (int e = 0; e < 4; ++e) {
-      prow[2 * e] = make_float4(acc[0][e], acc[1][e], acc[2][e], acc[3][e]);
-      prow[2 * e + 1] = make_float4(acc[4][e], acc[5][e], acc[6][e], acc[7][e]);
-    }
-    if (kg == 0) reinterpret_cast<float2*>(a.part_ml)[row] = make_float2(m_run, l_run);
+  for (int e = 0; e < 4; ++e) {
+    uint4 o;
+    o.x = pack_bf16x2(acc[0][e] * inv, acc[1][e] * inv);
+    o.y = pack_bf16x2(acc[2][e] * inv, acc[3][e] * inv);
+    o.z = pack_bf16x2(acc[4][e] * inv, acc[5][e] * inv);
+    o.w = pack_bf16x2(acc[6][e] * inv, acc[7][e] * inv);
+    orow[e] = o;
   }
+}
+
+// Unnormalised partial (D f32 per head) + (max, sum) to slot `slot` of the workspace.
+template <int D>
+__device__ __forceinline__ void write_partial(const DecodeArgs& a, int64_t slot, int kvh, int lane,
+                                              const f32x4 (&acc)[8], float m_run, float l_run) {
+  const int r = lane & 15, kg = lane >> 4;
+  if (r >= a.group || 32 * kg >= D) return;
+  const int64_t row = slot * a.num_heads + kvh * a.group + r;
+  float4* prow = reinterpret_cast<float4*>(a.part_o + row * D + 32 * kg);
+#pragma unroll
+  for (int e = 0; e < 4; ++e) {
+    prow[2 * e] = make_float4(acc[0][e], acc[1][e], acc[2][e], acc[3][e]);
+    prow[2 * e + 1] = make_float4(acc[4][e], acc[5][e], acc[6][e], acc[7][e]);
+  }
+  if (kg == 0) reinterpret_cast<float2*>(a.part_ml)[row] = make_float2(m_run, l_run);
+}
+
+// compute_segment, then: `direct` (the segment is the whole sequence) -> out,
+// otherwise -> partial slot `slot`.
+template <int D>
+__device__ __forceinline__ void run_segment(const DecodeArgs& a, uint4* lds, int b, int kvh,
+                                            int t0, int t1, int64_t slot, bool direct,
+                                            int lane) {
+  f32x4 acc[8];
+  float m_run, l_run;
+  compute_segment<D>(a, lds, b, kvh, t0, t1, lane, acc, m_run, l_run);
+  if (direct) write_output<D>(a, b, kvh, lane, acc, l_run);
+  else write_partial<D>(a, slot, kvh, lane, acc, m_run, l_run);
 }
 
 // Fixed-chunk split: grid.x = batch * max_chunks, grid.y = num_kv_heads / NW,
@@ -363,6 +387,77 @@ __global__ __launch_bounds__(NW * 64) void paged_decode_splitk_kernel(DecodeArgs
   const bool direct = ctx <= chunk;
   run_segment<D>(a, k_tile[wave], b, blockIdx.y * NW + wave, t0, t1,
                  (int64_t)b * max_chunks + c, direct, lane);
+}
+
+// Whole-sequence split: every sequence is finished inside one workgroup, so
+// there is no workspace and no second pass.  grid.x = batch * (num_kv_heads /
+// hpw), block = NW * 64.  Workgroup (b, head group hg) owns `hpw` KV heads of
+// sequence b; its NW waves are hpw heads x NW / hpw parts: wave w takes head
+// hg * hpw + w % hpw and the (w / hpw)-th of NW / hpw equal runs of the
+// sequence's 32-position steps.  The parts of a head meet through LDS (each
+// wave's K tile is free by then and exactly holds its 34 floats per lane) and
+// the wave of part 0 merges them and writes the output.  Meant for batches of
+// similar lengths: a workgroup's time follows its sequence's length.
+template <int NW, int D>
+__global__ __launch_bounds__(NW * 64) void paged_decode_whole_kernel(DecodeArgs a, int hpw) {
+  using H = HeadDim<D>;
+  __shared__ uint4 k_tile[NW][kStep * H::kLdsRowPieces];
+  constexpr int kLanesWithDims = D / 32 * 16;   // lanes whose k-group holds real dims
+  static_assert(sizeof(uint4) * kStep * H::kLdsRowPieces >= 34 * kLanesWithDims * sizeof(float),
+                "a wave's K tile must hold its partial");
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int lane = threadIdx.x & 63;
+  const int parts = NW / hpw;
+  const int groups = a.num_kv_heads / hpw;
+  const int b = blockIdx.x / groups;
+  const int hg = blockIdx.x - b * groups;
+  const int part = wave / hpw;
+  const int kvh = hg * hpw + (wave - part * hpw);
+  const int ctx = min(max(as_constant(a.context_lens)[b], 0), a.max_blocks * a.block_size);
+  const int steps = (ctx + kStep - 1) / kStep;
+  const int s0 = (int)((int64_t)part * steps / parts);
+  const int s1 = (int)((int64_t)(part + 1) * steps / parts);
+
+  f32x4 acc[8];
+#pragma unroll
+  for (int jd = 0; jd < 8; ++jd) acc[jd] = f32x4{0.f, 0.f, 0.f, 0.f};
+  float m_run = kNegBig, l_run = 0.f;
+  if (s1 > s0)
+    compute_segment<D>(a, k_tile[wave], b, kvh, s0 * kStep, min(ctx, s1 * kStep), lane, acc, m_run,
+                       l_run);
+  if (parts > 1) {
+    // value v of lane l at float v * kLanesWithDims + l of the wave's tile
+    const bool holds_dims = lane < kLanesWithDims;
+    __syncthreads();   // every wave is done reading its K tile
+    if (part > 0 && holds_dims) {
+      float* mine = reinterpret_cast<float*>(k_tile[wave]) + lane;
+#pragma unroll
+      for (int jd = 0; jd < 8; ++jd)
+#pragma unroll
+        for (int e = 0; e < 4; ++e) mine[(4 * jd + e) * kLanesWithDims] = acc[jd][e];
+      mine[32 * kLanesWithDims] = m_run;
+      mine[33 * kLanesWithDims] = l_run;
+    }
+    __syncthreads();
+    if (part > 0) return;
+    if (holds_dims) {
+      for (int p = 1; p < parts; ++p) {
+        const float* theirs = reinterpret_cast<const float*>(k_tile[wave + p * hpw]) + lane;
+        const float m_p = theirs[32 * kLanesWithDims], l_p = theirs[33 * kLanesWithDims];
+        const float m_new = fmaxf(m_run, m_p);
+        const float keep = __builtin_amdgcn_exp2f((m_run - m_new) * a.scale_log2e);
+        const float w = __builtin_amdgcn_exp2f((m_p - m_new) * a.scale_log2e);
+        m_run = m_new;
+        l_run = fmaf(l_run, keep, w * l_p);
+#pragma unroll
+        for (int jd = 0; jd < 8; ++jd)
+#pragma unroll
+          for (int e = 0; e < 4; ++e)
+            acc[jd][e] = fmaf(acc[jd][e], keep, w * theirs[(4 * jd + e) * kLanesWithDims]);
+      }
+    }
+  }
+  write_output<D>(a, b, kvh, lane, acc, l_run);
 }
 
 // Inclusive prefix sum over the 64 lanes of a wave with DPP moves: a
@@ -565,6 +660,15 @@ __global__ __launch_bounds__(kMaxHeadDim) void paged_decode_combine_kernel(
 
 int round_up(int x, int m) { return (x + m - 1) / m * m; }
 
+// Whole-sequence mode: KV heads per 8-wave workgroup.  As many as still give
+// one workgroup per CU (256), so that the split inside a workgroup is no finer
+// than needed; it must divide the number of KV heads.
+int whole_sequence_heads_per_workgroup(int64_t batch, int num_kv_heads) {
+  int hpw = 8;
+  while (hpw > 1 && (num_kv_heads % hpw != 0 || batch * (num_kv_heads / hpw) < 256)) hpw /= 2;
+  return hpw;
+}
+
 // Balanced mode launches at most one workgroup per CU of an MI355X, and never
 // gives a workgroup fewer than 4 steps (128 positions): below that the
 // partials cost more than the split gains.
@@ -625,6 +729,7 @@ extern "C" size_t nvj_paged_decode_workspace_bytes(int32_t batch, int32_t num_he
                                                    int32_t head_dim, int32_t max_blocks,
                                                    int32_t block_size, int32_t num_kv_heads,
                                                    int32_t chunk) {
+  if (chunk == NVJ_CHUNK_WHOLE_SEQUENCE) return 0;   // finished inside the workgroups
   if (batch <= 0 || num_heads <= 0 || (head_dim != 128 && head_dim != 64) || max_blocks <= 0 ||
       block_size <= 0 || num_kv_heads <= 0 || chunk < 0 || chunk % kStep != 0)
     return 0;
@@ -642,13 +747,14 @@ extern "C" int nvj_paged_decode_launch_phases(void* stream, const void* q, const
                                               int32_t block_size, int32_t max_blocks,
                                               int32_t num_blocks, float scale, int32_t chunk,
                                               uint32_t phases) {
+  const bool whole = chunk == NVJ_CHUNK_WHOLE_SEQUENCE;
   if (batch < 0 || num_heads <= 0 || num_kv_heads <= 0 || head_dim <= 0 || block_size <= 0 ||
-      max_blocks < 0 || num_blocks <= 0 || chunk < 0)
+      max_blocks < 0 || num_blocks <= 0 || (chunk < 0 && !whole))
     return NVJ_ERR_BAD_SHAPE;
   if (num_heads % num_kv_heads != 0) return NVJ_ERR_BAD_SHAPE;
   const int group = num_heads / num_kv_heads;
   if ((head_dim != 128 && head_dim != 64) || group > 16 || block_size % kStep != 0 ||
-      chunk % kStep != 0)
+      (!whole && chunk % kStep != 0))
     return NVJ_ERR_UNSUPPORTED;
   if ((int64_t)max_blocks * block_size > INT32_MAX) return NVJ_ERR_BAD_SHAPE;
   if (!(scale >= 0.f)) return NVJ_ERR_BAD_SHAPE;   // the running max assumes a non-negative scale
@@ -677,6 +783,16 @@ extern "C" int nvj_paged_decode_launch_phases(void* stream, const void* q, const
   a.max_blocks = max_blocks;
   a.num_blocks = num_blocks;
   a.scale_log2e = scale * kLog2e;
+
+  if (whole && max_blocks > 0) {
+    if ((int64_t)batch * num_kv_heads > INT32_MAX) return NVJ_ERR_BAD_SHAPE;
+    if (!(phases & NVJ_PHASE_SPLITK)) return NVJ_OK;   // there is no second pass
+    const int hpw = whole_sequence_heads_per_workgroup(batch, num_kv_heads);
+    const dim3 grid((unsigned)(batch * (num_kv_heads / hpw)));
+    if (head_dim == 128) paged_decode_whole_kernel<8, 128><<<grid, dim3(512), 0, s>>>(a, hpw);
+    else paged_decode_whole_kernel<8, 64><<<grid, dim3(512), 0, s>>>(a, hpw);
+    return hipGetLastError() == hipSuccess ? NVJ_OK : NVJ_ERR_LAUNCH;
+  }
 
   WorkspacePlan plan = {0, 1, 0, 0};
   int32_t* prefix = nullptr;

@@ -30,7 +30,8 @@ from .. import _lib
 from ..layers.activation import silu_and_mul
 from ..layers.attention import Attention
 from ..layers.layernorm import rms_norm
-from ..layers.paged_attention import paged_attention, paged_decode_workspace_bytes
+from ..layers.paged_attention import (choose_split, paged_attention,
+                                      paged_decode_workspace_bytes)
 from ..layers.prefill_attention import variable_length_attention_prefill
 from ..layers.qk_rope_store import qk_norm_rope_store
 from ..utils.context import AttentionContext, create_decode_context, create_prefill_context
@@ -256,7 +257,7 @@ class DecodeStepRunner:
                 else:
                     o = paged_attention(q, attn.k_cache, attn.v_cache, context.block_tables,
                                         context.context_lens, attn.scale, attn.block_size,
-                                        workspace=attn.workspace)
+                                        chunk=context.decode_split, workspace=attn.workspace)
                 h = F.linear(o.reshape(-1, qs), lw["o"])
                 h, residual = self._rms(h, lw["ln2"], residual)
                 h = F.linear(self._silu_mul(F.linear(h, lw["gate_up"])), lw["down"])
@@ -284,7 +285,9 @@ class DecodeStepRunner:
                                                   self.cfg.block_size)
         d = self.device
         t = lambda a: torch.from_numpy(a).to(d)
-        return t(ids), t(pos), create_decode_context(t(ctx), t(slots), t(bt))
+        # the lengths are host integers here, as in the reference's filler: pick the split
+        split = choose_split(ctx, self.cfg.num_kv_heads)
+        return t(ids), t(pos), create_decode_context(t(ctx), t(slots), t(bt), split)
 
     def make_prefill_inputs(self, token_lists, block_tables):
         ids, pos, cu, slots, max_len = prepare_prefill(token_lists, block_tables,

@@ -117,7 +117,7 @@ class Attention:
         q = q.to(self.k_cache.dtype)      # layers/attention.py:386-387
         return paged_attention(q, self.k_cache, self.v_cache, context.block_tables,
                                context.context_lens, self.scale, self.block_size,
-                               workspace=self.workspace)
+                               chunk=context.decode_split, workspace=self.workspace)
 
     def __call__(self, q, k, v, context: AttentionContext):
         if self.k_cache is None or self.v_cache is None:

@@ -13,7 +13,10 @@ import torch
 
 from .. import _lib
 
-__all__ = ["paged_attention", "paged_decode_workspace_bytes", "default_chunk"]
+__all__ = ["paged_attention", "paged_decode_workspace_bytes", "default_chunk", "WHOLE_SEQUENCE",
+           "choose_split"]
+
+WHOLE_SEQUENCE = _lib.NVJ_CHUNK_WHOLE_SEQUENCE
 
 
 def _require(cond: bool, msg: str) -> None:
@@ -45,6 +48,19 @@ def paged_decode_workspace_bytes(batch: int, num_heads: int, head_dim: int,
         batch, num_heads, head_dim, max_blocks, block_size, num_kv_heads, chunk))
 
 
+def choose_split(context_lens_host, num_kv_heads: int) -> int:
+    """``chunk`` for a batch whose lengths the host knows (the reference's filler
+    builds ``context_lens`` from Python ints, ``engine/model_runner.py:334-376``):
+    ``WHOLE_SEQUENCE`` when the sequences fill the GPU (``batch * num_kv_heads >=
+    256`` workgroup slots) and the longest is within 10 % of the mean, else 0
+    (balanced split)."""
+    lens = [int(n) for n in context_lens_host]
+    if not lens or len(lens) * num_kv_heads < 256:
+        return 0
+    mean = sum(lens) / len(lens)
+    return WHOLE_SEQUENCE if mean > 0 and max(lens) <= 1.1 * mean else 0
+
+
 def paged_attention(q, k_cache, v_cache, block_tables, context_lens, scale, block_size,
                     *, chunk: int = 0, out: torch.Tensor | None = None,
                     workspace: torch.Tensor | None = None,
@@ -61,7 +77,9 @@ def paged_attention(q, k_cache, v_cache, block_tables, context_lens, scale, bloc
 
     Returns [batch, num_heads, head_dim] bf16.  ``chunk`` (0 = balanced split
     derived from ``context_lens`` on the device; > 0 = that many positions per
-    workgroup, multiple of 32), ``out`` and ``workspace``
+    workgroup, multiple of 32; ``WHOLE_SEQUENCE`` = each sequence finished inside
+    one workgroup, no workspace and no combine launch, for batches of similar
+    lengths), ``out`` and ``workspace``
     (uint8 tensor of at least ``paged_decode_workspace_bytes`` bytes) are
     optional tuning/reuse knobs the reference does not have; ``phases`` selects
     the split-K launch, the combine launch or both (timing aid).

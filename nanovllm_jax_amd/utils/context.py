@@ -39,6 +39,12 @@ class AttentionContext:
                         -1 means "do not store".
     block_tables        [batch, max_blocks] int32, logical -> physical page,
                         padded with -1.
+    decode_split        how the decode kernel divides the positions of the batch
+                        (``chunk`` of ``paged_attention``): 0 = balanced on the
+                        device from ``context_lens``; the filler, which knows
+                        the lengths on the host, may ask for the whole-sequence
+                        mode instead (``layers.paged_attention.choose_split``).
+                        Not a field of the reference's dataclass.
     """
     is_prefill: bool = False
     cu_seqlens_q: Any = None
@@ -49,14 +55,16 @@ class AttentionContext:
     slot_mapping: Any = None
     block_tables: Any = None
     last_token_indices: Any = None
+    decode_split: int = 0
 
 
-def create_decode_context(context_lens, slot_mapping, block_tables) -> AttentionContext:
+def create_decode_context(context_lens, slot_mapping, block_tables,
+                          decode_split: int = 0) -> AttentionContext:
     """Context for one decode step (every token is a sequence's last token, so
     ``last_token_indices`` stays None)."""
     return AttentionContext(is_prefill=False, context_lens=context_lens,
                             slot_mapping=slot_mapping, block_tables=block_tables,
-                            last_token_indices=None)
+                            last_token_indices=None, decode_split=decode_split)
 
 
 def create_prefill_context(cu_seqlens_q, cu_seqlens_k, max_seqlen_q: int, max_seqlen_k: int,

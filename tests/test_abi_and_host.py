@@ -50,6 +50,7 @@ def test_argument_validation_without_a_gpu():
     assert call(Hq=256, Hkv=8) == -3       # group > 16
     assert call(bs=48) == -3
     assert call(chunk=100) == -3
+    assert call(chunk=-2) == -2                   # only -1 (whole sequence) is a mode below 0
     assert call(batch=-1) == -2
     assert call(batch=0) == 0              # empty batch: nothing to do
     assert call(ptr=0) == -1
@@ -145,3 +146,12 @@ def test_workload_metadata(name):
     if name == "C3":
         assert w.context_lens.min() >= 16 and w.context_lens.max() <= 32768
         assert w.num_blocks == int(np.ceil(1.1 * nblk.sum()))
+
+
+def test_choose_split_policy():
+    from nanovllm_jax_amd.layers.paged_attention import WHOLE_SEQUENCE, choose_split
+    assert choose_split([4096] * 64, 8) == WHOLE_SEQUENCE          # C2
+    assert choose_split([1024] * 128, 8) == WHOLE_SEQUENCE         # C5
+    assert choose_split([32768] * 16, 8) == 0                      # C4: too few workgroups
+    assert choose_split([16, 32768] * 128, 8) == 0                 # ragged
+    assert choose_split([], 8) == 0

@@ -24,7 +24,7 @@ def oracle(q, kc, vc, bt, ctx, scale, bs):
     return paged_decode_attention_per_seq_ref(q, kc, vc, bt, ctx, scale, bs)
 
 
-@pytest.mark.parametrize("chunk", [0, 32, 64, 256, 1024])
+@pytest.mark.parametrize("chunk", [0, 32, 64, 256, 1024, -1])
 @pytest.mark.parametrize("Hq,Hkv", [(16, 8), (32, 8), (64, 8), (8, 8), (8, 2), (4, 1)])
 def test_small_random(Hq, Hkv, chunk):
     print(f"case small_random Hq={Hq} Hkv={Hkv} chunk={chunk}", flush=True)
@@ -220,3 +220,69 @@ def test_d64_random_groups_and_tails(Hq, Hkv):
         got = run_hip(q, kc, vc, bt, ctx, scale, bs, chunk)
         assert_close_bf16(got, want, what=f"D=64 Hq={Hq} Hkv={Hkv} chunk={chunk}")
     assert np.array_equal(got[0], np.repeat(vc[bt[0, 0], 0], Hq // Hkv, axis=0))
+
+
+# ---- whole-sequence mode (chunk = -1): every sequence finished inside one workgroup ----
+@pytest.mark.parametrize("B,Hq,Hkv,D", [(3, 32, 8, 128),     # 1 head per workgroup, 8 parts
+                                        (64, 16, 8, 128),    # 2 heads x 4 parts
+                                        (128, 16, 8, 128),   # 4 heads x 2 parts
+                                        (260, 8, 8, 128),    # 8 heads, no split inside
+                                        (90, 12, 6, 128),    # 6 KV heads: 2 per workgroup
+                                        (70, 8, 4, 64),      # head_dim 64, 1 head x 8 parts
+                                        (140, 8, 4, 64),     # head_dim 64, 2 heads x 4 parts
+                                        (5, 4, 1, 128)])
+def test_whole_sequence_mode(B, Hq, Hkv, D):
+    """Lengths around the number of parts (fewer steps than parts, empty parts),
+    empty sequences, tails, several pages; compared with the oracle and with the
+    balanced split."""
+    print(f"case whole-sequence B={B} Hq={Hq} Hkv={Hkv} D={D}", flush=True)
+    rng = np.random.Generator(np.random.PCG64(900 + B + Hkv))
+    bs = 64
+    ctx = rng.integers(1, 400, size=B)
+    ctx[:min(B, 12)] = [0, 1, 31, 32, 33, 64, 65, 255, 256, 257, 300, 96][:min(B, 12)]
+    NB = int((-(-ctx // bs)).sum()) + 2
+    q, kc, vc, bt, ctx = make_problem(900 + B, B, Hq, Hkv, D, bs, NB, ctx)
+    scale = 1.0 / np.sqrt(D)
+    want = oracle(q, kc, vc, bt, ctx, scale, bs)
+    got = run_hip(q, kc, vc, bt, ctx, scale, bs, -1)
+    assert_close_bf16(got, want, what=f"whole-sequence B={B}")
+    assert not got[ctx == 0].any(), "ctx=0 must give zeros"
+    one = np.flatnonzero(ctx == 1)[0]
+    assert np.array_equal(got[one], np.repeat(vc[bt[one, 0], 0], Hq // Hkv, axis=0))
+    balanced = run_hip(q, kc, vc, bt, ctx, scale, bs, 0)
+    assert_close_bf16(got, balanced, what="whole-sequence vs balanced")
+
+
+def test_whole_sequence_mode_needs_no_workspace_and_ignores_garbage():
+    """workspace_bytes is 0, a NULL workspace is accepted, and nothing beyond
+    ctx or in padding table entries is read."""
+    print("case whole-sequence no workspace / garbage", flush=True)
+    import torch
+    from nanovllm_jax_amd import _lib
+    from nanovllm_jax_amd.layers.paged_attention import WHOLE_SEQUENCE, paged_decode_workspace_bytes
+    B, Hq, Hkv, D, bs, NB = 40, 32, 8, 128, 256, 200
+    assert paged_decode_workspace_bytes(B, Hq, D, 4, bs, Hkv, WHOLE_SEQUENCE) == 0
+    rng = np.random.Generator(np.random.PCG64(77))
+    ctx = rng.integers(200, 1000, size=B)
+    q, kc, vc, bt, ctx = make_problem(78, B, Hq, Hkv, D, bs, NB, ctx)
+    want = oracle(q, kc, vc, bt, ctx, 0.09, bs)
+    # poison: NaN patterns in every slot past ctx of the last live page, wild padding entries
+    kc2, vc2, bt2 = kc.copy(), vc.copy(), bt.copy()
+    for b in range(B):
+        pages = -(-int(ctx[b]) // bs)
+        tail = int(ctx[b]) - (pages - 1) * bs
+        kc2[bt[b, pages - 1], tail:] = 0x7FC0
+        vc2[bt[b, pages - 1], tail:] = 0x7FC0
+        bt2[b, pages:] = 2 ** 30
+    dev = "cuda:0"
+    lib = _lib.load()
+    qt, kt, vt = bits_to_torch(q, dev), bits_to_torch(kc2, dev), bits_to_torch(vc2, dev)
+    btt, ct = torch.from_numpy(bt2).to(dev), torch.from_numpy(ctx).to(dev)
+    out = torch.empty_like(qt)
+    code = lib.nvj_paged_decode_launch(
+        torch.cuda.current_stream().cuda_stream, qt.data_ptr(), kt.data_ptr(), vt.data_ptr(),
+        btt.data_ptr(), ct.data_ptr(), out.data_ptr(), None, 0, B, Hq, Hkv, D, bs, bt.shape[1],
+        NB, 0.09, WHOLE_SEQUENCE)
+    assert code == 0
+    torch.cuda.synchronize()
+    assert_close_bf16(torch_to_bits(out), want, what="whole-sequence, NULL workspace, poison")
