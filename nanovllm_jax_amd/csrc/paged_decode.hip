@@ -763,7 +763,7 @@ extern "C" int nvj_paged_decode_launch_phases(void* stream, const void* q, const
   if (max_blocks > 0 && !block_tables) return NVJ_ERR_NULL_POINTER;
   if ((reinterpret_cast<uintptr_t>(q) | reinterpret_cast<uintptr_t>(k_cache) |
        reinterpret_cast<uintptr_t>(v_cache) | reinterpret_cast<uintptr_t>(out) |
-       reinterpret_cast<uintptr_t>(workspace)) & 15u)
+       (whole ? 0 : reinterpret_cast<uintptr_t>(workspace))) & 15u)   // unused in whole mode
     return NVJ_ERR_WORKSPACE;
   hipStream_t s = static_cast<hipStream_t>(stream);
 

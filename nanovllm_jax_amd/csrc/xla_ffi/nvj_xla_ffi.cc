@@ -52,7 +52,8 @@ ffi::Error StoreKvcacheImpl(hipStream_t stream, ffi::AnyBuffer key, ffi::AnyBuff
 }
 
 // operands: q [B, Hq, D], k_cache, v_cache [NB, bs, Hkv, D] bf16, block_tables [B, MB],
-// context_lens [B] s32; attrs scale (f32), chunk (s32, 0 = balanced split);
+// context_lens [B] s32; attrs scale (f32), chunk (s32, 0 = balanced split, -1 = whole
+// sequence per workgroup: the workspace result is then unused);
 // results: out [B, Hq, D] bf16 and the workspace (u8, sized by
 // nvj_paged_decode_workspace_bytes on the Python side so that XLA owns it).
 ffi::Error PagedDecodeImpl(hipStream_t stream, ffi::Buffer<ffi::DataType::BF16> q,
