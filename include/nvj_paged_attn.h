@@ -103,6 +103,14 @@ NVJ_API int32_t nvj_paged_decode_default_chunk(int32_t batch, int32_t num_kv_hea
                                        int32_t max_blocks, int32_t block_size);
 
 /*
+ * Number of workgroups chunk == NVJ_CHUNK_WHOLE_SEQUENCE launches for a batch:
+ * batch * num_kv_heads / (KV heads per workgroup).  One 8-wave workgroup is
+ * resident per CU (256 on MI355X), so that mode pays off when this is (just
+ * under) a multiple of 256 and the lengths are similar; 0 on invalid arguments.
+ */
+NVJ_API int32_t nvj_paged_decode_whole_sequence_workgroups(int32_t batch, int32_t num_kv_heads);
+
+/*
  * Bytes of device workspace nvj_paged_decode_launch needs for the partials
  * (fp32 accumulators plus running max and sum per partial; in balanced mode
  * also batch + 1 int32 prefix sums) for the given `chunk` mode.  Returns 0 on

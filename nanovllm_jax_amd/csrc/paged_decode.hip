@@ -725,6 +725,12 @@ extern "C" int32_t nvj_paged_decode_default_chunk(int32_t batch, int32_t num_kv_
   return round_up((int)chunk, kStep);
 }
 
+extern "C" int32_t nvj_paged_decode_whole_sequence_workgroups(int32_t batch,
+                                                               int32_t num_kv_heads) {
+  if (batch <= 0 || num_kv_heads <= 0 || (int64_t)batch * num_kv_heads > INT32_MAX) return 0;
+  return batch * (num_kv_heads / whole_sequence_heads_per_workgroup(batch, num_kv_heads));
+}
+
 extern "C" size_t nvj_paged_decode_workspace_bytes(int32_t batch, int32_t num_heads,
                                                    int32_t head_dim, int32_t max_blocks,
                                                    int32_t block_size, int32_t num_kv_heads,

@@ -51,14 +51,18 @@ def paged_decode_workspace_bytes(batch: int, num_heads: int, head_dim: int,
 def choose_split(context_lens_host, num_kv_heads: int) -> int:
     """``chunk`` for a batch whose lengths the host knows (the reference's filler
     builds ``context_lens`` from Python ints, ``engine/model_runner.py:334-376``):
-    ``WHOLE_SEQUENCE`` when the sequences fill the GPU (``batch * num_kv_heads >=
-    256`` workgroup slots) and the longest is within 10 % of the mean, else 0
-    (balanced split)."""
+    ``WHOLE_SEQUENCE`` when the longest sequence is within 10 % of the mean and
+    the workgroups of that mode fill whole rounds of the 256 CUs to at least
+    95 % (one 8-wave workgroup is resident per CU), else 0 (balanced split)."""
     lens = [int(n) for n in context_lens_host]
-    if not lens or len(lens) * num_kv_heads < 256:
+    if not lens:
         return 0
     mean = sum(lens) / len(lens)
-    return WHOLE_SEQUENCE if mean > 0 and max(lens) <= 1.1 * mean else 0
+    if mean <= 0 or max(lens) > 1.1 * mean:
+        return 0
+    wgs = int(_lib.load().nvj_paged_decode_whole_sequence_workgroups(len(lens), num_kv_heads))
+    rounds = -(-wgs // 256)
+    return WHOLE_SEQUENCE if wgs > 0 and wgs >= 0.95 * rounds * 256 else 0
 
 
 def paged_attention(q, k_cache, v_cache, block_tables, context_lens, scale, block_size,

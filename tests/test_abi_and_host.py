@@ -155,3 +155,7 @@ def test_choose_split_policy():
     assert choose_split([32768] * 16, 8) == 0                      # C4: too few workgroups
     assert choose_split([16, 32768] * 128, 8) == 0                 # ragged
     assert choose_split([], 8) == 0
+    assert choose_split([2048] * 40, 8) == 0       # 320 workgroups: a second round at 25 %
+    assert choose_split([2048] * 96, 8) == 0       # 384 workgroups
+    assert choose_split([2048] * 250, 8) == WHOLE_SEQUENCE         # 250 of 256
+    assert choose_split([2048] * 4096, 8) == WHOLE_SEQUENCE        # 16 full rounds
