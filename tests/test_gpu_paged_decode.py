@@ -286,3 +286,49 @@ def test_whole_sequence_mode_needs_no_workspace_and_ignores_garbage():
     assert code == 0
     torch.cuda.synchronize()
     assert_close_bf16(torch_to_bits(out), want, what="whole-sequence, NULL workspace, poison")
+
+
+@pytest.mark.parametrize("chunk", [0, -1])
+def test_decode_call_replays_in_a_hip_graph(chunk):
+    """The decode launch(es) captured once and replayed with the lengths and the
+    query updated in place between replays give what eager calls give, every
+    time (balanced split + combine, and the one-launch whole-sequence split)."""
+    print(f"case decode graph replays chunk={chunk}", flush=True)
+    import torch
+    from nanovllm_jax_amd import paged_attention
+    from nanovllm_jax_amd.layers.paged_attention import paged_decode_workspace_bytes
+    B, Hq, Hkv, D, bs, NB = 48, 32, 8, 128, 64, 400
+    rng = np.random.Generator(np.random.PCG64(4242))
+    ctx0 = rng.integers(100, 500, size=B)
+    q, kc, vc, bt, ctx0 = make_problem(4243, B, Hq, Hkv, D, bs, NB, ctx0)
+    dev = "cuda:0"
+    qt, kt, vt = bits_to_torch(q, dev), bits_to_torch(kc, dev), bits_to_torch(vc, dev)
+    btt, ct = torch.from_numpy(bt).to(dev), torch.from_numpy(ctx0).to(dev)
+    out = torch.empty_like(qt)
+    ws = torch.empty(max(16, paged_decode_workspace_bytes(B, Hq, D, bt.shape[1], bs, Hkv, chunk)),
+                     dtype=torch.uint8, device=dev)
+    call = lambda: paged_attention(qt, kt, vt, btt, ct, 0.088, bs, chunk=chunk, out=out,
+                                   workspace=ws)
+    s = torch.cuda.Stream(dev)
+    s.wait_stream(torch.cuda.current_stream(dev))
+    with torch.cuda.stream(s):
+        call()
+    torch.cuda.current_stream(dev).wait_stream(s)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        call()
+    for step in range(4):
+        # shorter lengths every replay (always inside the pages each sequence owns)
+        new_ctx = np.maximum(1, ctx0 - 37 * step).astype(np.int32)
+        ct.copy_(torch.from_numpy(new_ctx).to(dev))
+        qt.copy_(bits_to_torch(np.roll(q, step, axis=0), dev))
+        graph.replay()
+        torch.cuda.synchronize()
+        replayed = torch_to_bits(out).copy()
+        out.zero_()
+        call()                                   # eager, same inputs
+        torch.cuda.synchronize()
+        assert np.array_equal(replayed, torch_to_bits(out)), f"replay {step} differs from eager"
+        want = oracle(np.roll(q, step, axis=0), kc, vc, bt, new_ctx, 0.088, bs)
+        assert_close_bf16(replayed, want, what=f"graph replay {step}")
