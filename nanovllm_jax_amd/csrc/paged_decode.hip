@@ -264,13 +264,23 @@ __device__ __forceinline__ void compute_segment(const DecodeArgs& a, uint4* lds,
     const float mneg = -m_new * scale_log2e;
     m_run = m_new;
     float p0[4], p1[4];
-    float psum = 0.f;
 #pragma unroll
     for (int e = 0; e < 4; ++e) {
       p0[e] = __builtin_amdgcn_exp2f(fmaf(s0[e], scale_log2e, mneg));
       p1[e] = __builtin_amdgcn_exp2f(fmaf(s1[e], scale_log2e, mneg));
-      psum += p0[e] + p1[e];
     }
+    if (nvalid < kStep) {
+      // positions past the end weigh exactly 0 whatever the scale (at scale 0
+      // the exponential of a masked score is 1, not 0)
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        if (4 * kg + e >= nvalid) p0[e] = 0.f;
+        if (16 + 4 * kg + e >= nvalid) p1[e] = 0.f;
+      }
+    }
+    float psum = 0.f;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) psum += p0[e] + p1[e];
     l_run = fmaf(l_run, alpha, psum);
     uint4 pbits;
     pbits.x = pack_bf16x2(p0[0], p0[1]);

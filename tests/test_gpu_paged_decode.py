@@ -332,3 +332,21 @@ def test_decode_call_replays_in_a_hip_graph(chunk):
         assert np.array_equal(replayed, torch_to_bits(out)), f"replay {step} differs from eager"
         want = oracle(np.roll(q, step, axis=0), kc, vc, bt, new_ctx, 0.088, bs)
         assert_close_bf16(replayed, want, what=f"graph replay {step}")
+
+
+@pytest.mark.parametrize("chunk", [0, 64, -1])
+def test_scale_zero_gives_the_mean_of_v_over_the_live_positions(chunk):
+    """softmax of all-zero scores is uniform over the positions below ctx, and
+    positions past the end of a partly filled 32-position step must weigh
+    exactly 0 there too (the exponential of a masked score times scale 0 is 1)."""
+    print(f"case scale 0 chunk={chunk}", flush=True)
+    from oracle.paged_attention_oracle import bf16_bits_to_f32
+    B, Hq, Hkv, D, bs, NB = 6, 16, 8, 128, 64, 30
+    ctx = [1, 5, 33, 70, 100, 191]
+    q, kc, vc, bt, ctx = make_problem(55, B, Hq, Hkv, D, bs, NB, ctx)
+    got = bf16_bits_to_f32(run_hip(q, kc, vc, bt, ctx, 0.0, bs, chunk))
+    v = bf16_bits_to_f32(vc).astype(np.float64)
+    for b in range(B):
+        rows = np.concatenate([v[bt[b, p]] for p in range(-(-int(ctx[b]) // bs))])[:ctx[b]]
+        mean = np.repeat(rows.mean(axis=0), Hq // Hkv, axis=0)          # [Hq, D]
+        assert np.all(np.abs(got[b] - mean) <= 1e-2 + 1e-2 * np.abs(mean)), f"sequence {b}"

@@ -1,0 +1,93 @@
+"""Seeded random sweeps of the decode and prefill kernels against the CPU oracle:
+shapes, group sizes, page sizes, lengths and split modes that the hand-picked
+cases do not name (atol/rtol 1e-2 through the C ABI)."""
+import numpy as np
+import pytest
+
+from helpers import assert_close_bf16, bits_to_torch, make_problem, torch_to_bits
+
+pytestmark = pytest.mark.gpu
+
+
+def _decode_case(rng):
+    Hkv = int(rng.choice([1, 2, 3, 4, 5, 6, 7, 8, 12, 16]))
+    G = int(rng.choice([1, 2, 3, 4, 5, 7, 8, 16]))
+    D = int(rng.choice([128, 128, 64]))
+    bs = int(rng.choice([32, 64, 96, 160, 256]))
+    B = int(rng.choice([1, 2, 7, 33, 65, 130]))
+    if B * Hkv * G > 4096:           # keep the CPU oracle quick
+        B = max(1, 4096 // (Hkv * G))
+    kind = int(rng.integers(0, 3))
+    if kind == 0:
+        ctx = rng.integers(0, 3 * bs, size=B)
+    elif kind == 1:
+        ctx = rng.integers(1, 40, size=B)
+    else:
+        ctx = np.full(B, int(rng.integers(1, 700)))
+    ctx[rng.integers(0, B)] = int(rng.choice([0, 1, 31, 32, 33, bs, bs + 1]))
+    chunk = int(rng.choice([0, 0, -1, -1, 32, 96, 512]))
+    scale = float(rng.choice([D ** -0.5, 0.0, 0.3]))
+    gain = float(rng.choice([1.0, 1.0, 4.0]))
+    return dict(B=B, Hq=Hkv * G, Hkv=Hkv, D=D, bs=bs, ctx=ctx, chunk=chunk, scale=scale, gain=gain)
+
+
+@pytest.mark.parametrize("seed", range(40))
+def test_decode_random_case(seed):
+    import torch
+    from nanovllm_jax_amd import paged_attention
+    from oracle.paged_attention_oracle import paged_decode_attention_per_seq_ref
+    c = _decode_case(np.random.Generator(np.random.PCG64(31000 + seed)))
+    print(f"case decode sweep seed={seed} " +
+          " ".join(f"{k}={v}" for k, v in c.items() if k != "ctx") +
+          f" ctx={c['ctx'].min()}..{c['ctx'].max()}", flush=True)
+    NB = int((-(-c["ctx"] // c["bs"])).sum()) + 2
+    q, kc, vc, bt, ctx = make_problem(32000 + seed, c["B"], c["Hq"], c["Hkv"], c["D"], c["bs"], NB,
+                                      c["ctx"], q_gain=c["gain"])
+    dev = "cuda:0"
+    out = paged_attention(bits_to_torch(q, dev), bits_to_torch(kc, dev), bits_to_torch(vc, dev),
+                          torch.from_numpy(bt).to(dev), torch.from_numpy(ctx).to(dev), c["scale"],
+                          c["bs"], chunk=c["chunk"])
+    torch.cuda.synchronize()
+    want = paged_decode_attention_per_seq_ref(q, kc, vc, bt, ctx, c["scale"], c["bs"])
+    got = torch_to_bits(out)
+    assert_close_bf16(got, want, what=f"decode sweep seed={seed}")
+    assert not got[ctx == 0].any()
+
+
+def _prefill_case(rng):
+    Hkv = int(rng.choice([1, 2, 4, 8]))
+    G = int(rng.choice([1, 2, 4, 8]))
+    n = int(rng.integers(1, 7))
+    lens_q = [int(x) for x in rng.choice([0, 1, 2, 31, 32, 33, 127, 128, 129, 200, 257, 400], n)]
+    if rng.integers(0, 3) == 0:      # k shorter or longer than q for some sequences
+        lens_k = [max(0, x + int(rng.integers(-40, 41))) for x in lens_q]
+    else:
+        lens_k = list(lens_q)
+    if sum(lens_q) == 0:
+        lens_q[0] = lens_k[0] = 5
+    scale = float(rng.choice([128 ** -0.5, 0.0, 0.25]))
+    gain = float(rng.choice([1.0, 3.0]))
+    return dict(Hq=Hkv * G, Hkv=Hkv, lens_q=lens_q, lens_k=lens_k, scale=scale, gain=gain)
+
+
+@pytest.mark.parametrize("seed", range(24))
+def test_prefill_random_case(seed):
+    import torch
+    from nanovllm_jax_amd import variable_length_attention_prefill
+    from nanovllm_jax_amd.workloads import draw_bf16_bits
+    from oracle.paged_attention_oracle import variable_length_attention_prefill_ref
+    c = _prefill_case(np.random.Generator(np.random.PCG64(41000 + seed)))
+    print(f"case prefill sweep seed={seed} {c}", flush=True)
+    rng = np.random.Generator(np.random.PCG64(42000 + seed))
+    cu_q = np.concatenate([[0], np.cumsum(c["lens_q"])]).astype(np.int32)
+    cu_k = np.concatenate([[0], np.cumsum(c["lens_k"])]).astype(np.int32)
+    q = draw_bf16_bits(rng, (int(cu_q[-1]), c["Hq"], 128), c["gain"])
+    k = draw_bf16_bits(rng, (max(int(cu_k[-1]), 1), c["Hkv"], 128))
+    v = draw_bf16_bits(rng, (max(int(cu_k[-1]), 1), c["Hkv"], 128))
+    dev = "cuda:0"
+    out = variable_length_attention_prefill(
+        bits_to_torch(q, dev), bits_to_torch(k, dev), bits_to_torch(v, dev),
+        torch.from_numpy(cu_q).to(dev), torch.from_numpy(cu_k).to(dev), scale=c["scale"])
+    torch.cuda.synchronize()
+    want = variable_length_attention_prefill_ref(q, k, v, cu_q, cu_k, c["scale"])
+    assert_close_bf16(torch_to_bits(out), want, what=f"prefill sweep seed={seed}")
