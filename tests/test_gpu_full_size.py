@@ -8,7 +8,7 @@ import sys
 import numpy as np
 import pytest
 
-from helpers import assert_close_bf16, torch_to_bits
+from helpers import assert_close_bf16, bits_to_torch, torch_to_bits
 
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 if ROOT not in sys.path:
@@ -61,3 +61,61 @@ def test_c3_ragged_batch():
     w, outs, want = _run("C3", [0, 512])
     # sequences whose last page is partial must be present in this workload
     assert (w.context_lens % w.block_size != 0).sum() > w.batch // 2
+
+
+def test_pool_larger_than_4_gib_per_tensor():
+    """Pages near the top of a 5 GiB-per-tensor pool: every byte offset into the
+    caches needs more than 32 bits (decode reads, plain store, fused store)."""
+    print("case large pool addressing", flush=True)
+    import torch
+    from nanovllm_jax_amd import paged_attention, store_kv_to_cache
+    from oracle.paged_attention_oracle import (f32_to_bf16_bits, paged_decode_attention_per_seq_ref,
+                                               store_kv_to_cache_ref)
+    from nanovllm_jax_amd.workloads import draw_bf16_bits
+    dev = "cuda:0"
+    NB, bs, Hkv, D, Hq, B = 10240, 256, 8, 128, 32, 4          # 10240 pages x 512 KiB = 5 GiB
+    kc = torch.zeros((NB, bs, Hkv, D), dtype=torch.bfloat16, device=dev)
+    vc = torch.zeros((NB, bs, Hkv, D), dtype=torch.bfloat16, device=dev)
+    rng = np.random.Generator(np.random.PCG64(99))
+    ctx = np.array([700, 256, 1, 513], np.int32)
+    pages = [NB - 1 - i for i in range(8)]                      # all above the 4 GiB mark
+    bt = np.full((B, 3), -1, np.int32)
+    small_k = np.zeros((8, bs, Hkv, D), np.uint16)              # host copy of just those pages
+    small_v = np.zeros((8, bs, Hkv, D), np.uint16)
+    remap, nxt = {}, 0
+    for b in range(B):
+        for p in range(-(-int(ctx[b]) // bs)):
+            page = pages[nxt]
+            bt[b, p] = page
+            remap[page] = nxt
+            small_k[nxt] = draw_bf16_bits(rng, (bs, Hkv, D))
+            small_v[nxt] = draw_bf16_bits(rng, (bs, Hkv, D))
+            kc[page] = bits_to_torch(small_k[nxt], dev)
+            vc[page] = bits_to_torch(small_v[nxt], dev)
+            nxt += 1
+    q = draw_bf16_bits(rng, (B, Hq, D))
+    # store one new row per sequence at its last position, then read
+    k_new = rng.standard_normal((B, Hkv, D), dtype=np.float32)
+    v_new = draw_bf16_bits(rng, (B, Hkv, D))
+    slots = np.array([bt[b, (ctx[b] - 1) // bs] * bs + (ctx[b] - 1) % bs for b in range(B)], np.int64)
+    assert slots.min() * Hkv * D * 2 > 2 ** 32
+    store_kv_to_cache(torch.from_numpy(k_new).to(dev), bits_to_torch(v_new, dev),
+                      kc.view(-1, Hkv, D), vc.view(-1, Hkv, D),
+                      torch.from_numpy(slots.astype(np.int32)).to(dev))
+    small_bt = np.vectorize(lambda x: remap.get(int(x), -1))(bt).astype(np.int32)
+    small_slots = np.array([small_bt[b, (ctx[b] - 1) // bs] * bs + (ctx[b] - 1) % bs
+                            for b in range(B)], np.int32)
+    wk, wv = store_kv_to_cache_ref(k_new, v_new, small_k.reshape(-1, Hkv, D),
+                                   small_v.reshape(-1, Hkv, D), small_slots, negative_slots="skip")
+    for page, i in remap.items():
+        assert np.array_equal(torch_to_bits(kc[page]), wk.reshape(8, bs, Hkv, D)[i])
+        assert np.array_equal(torch_to_bits(vc[page]), wv.reshape(8, bs, Hkv, D)[i])
+    want = paged_decode_attention_per_seq_ref(q, wk.reshape(8, bs, Hkv, D), wv.reshape(8, bs, Hkv, D),
+                                              small_bt, ctx, D ** -0.5, bs)
+    for chunk in (0, 256, -1):
+        out = paged_attention(bits_to_torch(q, dev), kc, vc, torch.from_numpy(bt).to(dev),
+                              torch.from_numpy(ctx).to(dev), D ** -0.5, bs, chunk=chunk)
+        torch.cuda.synchronize()
+        assert_close_bf16(torch_to_bits(out), want, what=f"large pool chunk={chunk}")
+    del kc, vc
+    torch.cuda.empty_cache()
