@@ -58,16 +58,42 @@ __global__ __launch_bounds__(256) void add_rms_norm_kernel(
   const int lane = threadIdx.x & 63;
   const int64_t row = (int64_t)token * row_pieces;
 
+  // every load of the row is issued before the first store: residual_out may be
+  // the residual buffer itself, so a store would otherwise fence the loads
+  // that follow it
+  uint4 xv[PIECES], rv[PIECES];
+#pragma unroll
+  for (int j = 0; j < PIECES; ++j) {
+    const int p = lane + 64 * j;
+    if (p < row_pieces) {
+      xv[j] = x[row + p];
+      if (RESIDUAL) rv[j] = residual[row + p];
+    }
+  }
+  // short rows: the weights too, ahead of the reduction
+  constexpr bool kEarlyWeights = PIECES <= 2;
+  float4 wv[kEarlyWeights ? PIECES : 1][2];
+  if (kEarlyWeights) {
+#pragma unroll
+    for (int j = 0; j < PIECES; ++j) {
+      const int p = lane + 64 * j;
+      if (p < row_pieces) {
+        wv[j][0] = reinterpret_cast<const float4*>(weight)[2 * p];
+        wv[j][1] = reinterpret_cast<const float4*>(weight)[2 * p + 1];
+      }
+    }
+  }
+
   float s[PIECES][8];
   float a = 0.f;
 #pragma unroll
   for (int j = 0; j < PIECES; ++j) {
     const int p = lane + 64 * j;
     if (p < row_pieces) {
-      unpack8(x[row + p], s[j]);
+      unpack8(xv[j], s[j]);
       if (RESIDUAL) {
         float rs[8];
-        unpack8(residual[row + p], rs);
+        unpack8(rv[j], rs);
 #pragma unroll
         for (int e = 0; e < 8; ++e) s[j][e] = s[j][e] + rs[e];
         uint4 o;
@@ -88,8 +114,10 @@ __global__ __launch_bounds__(256) void add_rms_norm_kernel(
   for (int j = 0; j < PIECES; ++j) {
     const int p = lane + 64 * j;
     if (p < row_pieces) {
-      const float4 w0 = reinterpret_cast<const float4*>(weight)[2 * p];
-      const float4 w1 = reinterpret_cast<const float4*>(weight)[2 * p + 1];
+      const float4 w0 =
+          kEarlyWeights ? wv[kEarlyWeights ? j : 0][0] : reinterpret_cast<const float4*>(weight)[2 * p];
+      const float4 w1 = kEarlyWeights ? wv[kEarlyWeights ? j : 0][1]
+                                      : reinterpret_cast<const float4*>(weight)[2 * p + 1];
       uint4 o;
       o.x = pack2(s[j][0] * r * w0.x, s[j][1] * r * w0.y);
       o.y = pack2(s[j][2] * r * w0.z, s[j][3] * r * w0.w);
