@@ -206,7 +206,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
-    ap.add_argument("--workload", default="C2", choices=["C1", "C2", "C3", "C4", "C5"])
+    ap.add_argument("--workload", default="C2", choices=["C1", "C2", "C3", "C4", "C5", "R1"])
     ap.add_argument("--chunk", type=int, default=None,
                     help="split mode: 0 = balanced, > 0 = positions per workgroup, -1 = whole "
                          "sequence per workgroup; default: what the host filler would pick from "

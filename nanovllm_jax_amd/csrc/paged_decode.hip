@@ -685,10 +685,22 @@ int whole_sequence_heads_per_workgroup(int64_t batch, int num_kv_heads) {
 constexpr int kMaxBalancedWorkgroups = 256;
 constexpr int kMinBalancedSteps = 4;
 
-int balanced_workgroups(int64_t batch, int64_t max_blocks, int64_t block_size) {
+// Waves per workgroup = KV heads a workgroup covers: the largest of 8, 4, 2, 1
+// that divides the number of KV heads.
+int waves_per_workgroup(int num_kv_heads) {
+  return num_kv_heads % 8 == 0 ? 8 : num_kv_heads % 4 == 0 ? 4 : num_kv_heads % 2 == 0 ? 2 : 1;
+}
+
+// Runs (grid.x) of the balanced split.  grid.y = num_kv_heads / waves per
+// workgroup head groups walk the same runs, so the cap of one workgroup per CU
+// applies to their product.
+int balanced_workgroups(int64_t batch, int64_t max_blocks, int64_t block_size, int num_kv_heads) {
+  const int head_groups = num_kv_heads / waves_per_workgroup(num_kv_heads);
+  const int64_t cap = kMaxBalancedWorkgroups / head_groups > 0
+                          ? kMaxBalancedWorkgroups / head_groups : 1;
   const int64_t max_steps = batch * ((max_blocks * block_size + kStep - 1) / kStep);
   const int64_t wgs = (max_steps + kMinBalancedSteps - 1) / kMinBalancedSteps;
-  return (int)(wgs < 1 ? 1 : wgs > kMaxBalancedWorkgroups ? kMaxBalancedWorkgroups : wgs);
+  return (int)(wgs < 1 ? 1 : wgs > cap ? cap : wgs);
 }
 
 // Workspace layout.  Fixed chunks: slots = batch * max_chunks.  Balanced:
@@ -701,9 +713,9 @@ struct WorkspacePlan {
 };
 
 bool plan_workspace(int64_t batch, int64_t num_heads, int64_t head_dim, int64_t max_blocks,
-                    int64_t block_size, int chunk, WorkspacePlan* plan) {
+                    int64_t block_size, int num_kv_heads, int chunk, WorkspacePlan* plan) {
   if (chunk == 0) {
-    plan->num_wgs = balanced_workgroups(batch, max_blocks, block_size);
+    plan->num_wgs = balanced_workgroups(batch, max_blocks, block_size, num_kv_heads);
     plan->max_chunks = 0;
     plan->slots = plan->num_wgs + batch;
     const size_t floats = (size_t)plan->slots * num_heads * (head_dim + 2);
@@ -750,7 +762,9 @@ extern "C" size_t nvj_paged_decode_workspace_bytes(int32_t batch, int32_t num_he
       block_size <= 0 || num_kv_heads <= 0 || chunk < 0 || chunk % kStep != 0)
     return 0;
   WorkspacePlan plan;
-  if (!plan_workspace(batch, num_heads, head_dim, max_blocks, block_size, chunk, &plan)) return 0;
+  if (!plan_workspace(batch, num_heads, head_dim, max_blocks, block_size, num_kv_heads, chunk,
+                      &plan))
+    return 0;
   return plan.bytes;
 }
 
@@ -813,7 +827,8 @@ extern "C" int nvj_paged_decode_launch_phases(void* stream, const void* q, const
   WorkspacePlan plan = {0, 1, 0, 0};
   int32_t* prefix = nullptr;
   if (max_blocks > 0) {
-    if (!plan_workspace(batch, num_heads, head_dim, max_blocks, block_size, chunk, &plan))
+    if (!plan_workspace(batch, num_heads, head_dim, max_blocks, block_size, num_kv_heads, chunk,
+                        &plan))
       return NVJ_ERR_BAD_SHAPE;
     if (!workspace || workspace_bytes < plan.bytes) return NVJ_ERR_WORKSPACE;
     a.part_o = static_cast<float*>(workspace);
@@ -821,8 +836,7 @@ extern "C" int nvj_paged_decode_launch_phases(void* stream, const void* q, const
     if (chunk == 0) prefix = reinterpret_cast<int32_t*>(a.part_ml + plan.slots * num_heads * 2);
 
     if (phases & NVJ_PHASE_SPLITK) {
-      const int nw =
-          num_kv_heads % 8 == 0 ? 8 : num_kv_heads % 4 == 0 ? 4 : num_kv_heads % 2 == 0 ? 2 : 1;
+      const int nw = waves_per_workgroup(num_kv_heads);
       const unsigned gy = (unsigned)(num_kv_heads / nw);
       // one instantiation per (waves per workgroup, head_dim)
 #define NVJ_FOR_SHAPE(LAUNCH)                 \

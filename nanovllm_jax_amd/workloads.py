@@ -111,6 +111,15 @@ def make_workload(name: str, seed: int | None = None) -> DecodeWorkload:
         ctx = np.full(B, 1024, dtype=np.int32)
         bt = rng.permutation(NB).astype(np.int32).reshape(B, MB)
         gain = 1.0
+    elif name == "R1":   # the shape the reference itself times (profile_attention.py:19-34)
+        # MHA cache (32 KV heads), identity block tables, context lengths uniform in
+        # [200, 2048); the reference draws fp16 with jax.random, here bf16 from this seed
+        seed = 1101 if seed is None else seed
+        rng = np.random.Generator(np.random.PCG64(seed))
+        B, Hq, Hkv, D, bs, NB, MB = 64, 32, 32, 128, 256, 512, 8
+        ctx = rng.integers(200, 2048, size=B).astype(np.int32)
+        bt = np.arange(NB, dtype=np.int32).reshape(B, MB)
+        gain = 1.0
     else:
         raise KeyError(name)
     return DecodeWorkload(name=name, batch=B, num_heads=Hq, num_kv_heads=Hkv,
@@ -119,7 +128,7 @@ def make_workload(name: str, seed: int | None = None) -> DecodeWorkload:
                           slot_mapping=_slots(bt, ctx, bs), q_gain=gain, seed=seed)
 
 
-WORKLOADS = ("C1", "C2", "C3", "C4", "C5")
+WORKLOADS = ("C1", "C2", "C3", "C4", "C5", "R1")
 
 
 def draw_bf16_bits(rng: np.random.Generator, shape, gain: float = 1.0) -> np.ndarray:

@@ -159,3 +159,13 @@ def test_choose_split_policy():
     assert choose_split([2048] * 96, 8) == 0       # 384 workgroups
     assert choose_split([2048] * 250, 8) == WHOLE_SEQUENCE         # 250 of 256
     assert choose_split([2048] * 4096, 8) == WHOLE_SEQUENCE        # 16 full rounds
+
+
+def test_reference_profile_shape_workload():
+    """R1 restates the inputs of the reference's own timing script
+    (profile_attention.py:19-34): MHA cache, identity tables, lengths in [200, 2048)."""
+    from nanovllm_jax_amd.workloads import make_workload
+    w = make_workload("R1")
+    assert (w.batch, w.num_heads, w.num_kv_heads, w.head_dim, w.block_size) == (64, 32, 32, 128, 256)
+    assert np.array_equal(w.block_tables, np.arange(512, dtype=np.int32).reshape(64, 8))
+    assert w.context_lens.min() >= 200 and w.context_lens.max() < 2048
