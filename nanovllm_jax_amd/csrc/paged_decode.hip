@@ -10,7 +10,10 @@
 // dim] layout).  A wave owns the G query heads of its KV head, so every K/V
 // byte is fetched once per group.  The runs are either equal cuts of all the
 // steps of the batch, derived on the device from context_lens (balanced split,
-// the default), or fixed chunks of each sequence.
+// the default), or fixed chunks of each sequence.  A third mode finishes every
+// sequence inside one workgroup (its waves are a few KV heads x equal parts of
+// the sequence, merged through LDS): one launch, no workspace, for batches of
+// similar lengths.
 //
 // Inner step = 32 positions of one page:
 //   * K: 8 x 16-byte loads per lane, quarter-wave = one 256-byte (position,
@@ -26,9 +29,9 @@
 //   * O^T[dim, qhead] += V^T . P^T with 8 MFMAs.
 // Loads for step i+1 are issued before the arithmetic of step i.
 //
-// The partial (unnormalised O, running max, running sum) of every segment goes
-// to the workspace; the combine kernel merges the segments of a sequence.  A
-// sequence that is one segment is written directly.
+// In the first two modes the partial (unnormalised O, running max, running
+// sum) of every segment goes to the workspace and the combine kernel merges the
+// segments of a sequence; a sequence that is one segment is written directly.
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
