@@ -89,5 +89,16 @@ def test_prefill_random_case(seed):
         bits_to_torch(q, dev), bits_to_torch(k, dev), bits_to_torch(v, dev),
         torch.from_numpy(cu_q).to(dev), torch.from_numpy(cu_k).to(dev), scale=c["scale"])
     torch.cuda.synchronize()
+    got = torch_to_bits(out)
     want = variable_length_attention_prefill_ref(q, k, v, cu_q, cu_k, c["scale"])
-    assert_close_bf16(torch_to_bits(out), want, what=f"prefill sweep seed={seed}")
+    assert_close_bf16(got, want, what=f"prefill sweep seed={seed}")
+    # Also against the exact float64 softmax.  The oracle above rounds the
+    # probabilities to bf16 as the reference's attention does, the kernel rounds
+    # its own (differently scaled) ones: two independent roundings.  Over 2000
+    # further seeds of this generator five cases had one element outside the bar
+    # against that oracle, by at most 1.3e-3, while the kernel itself stayed at
+    # least 2.6e-3 inside it against float64; this is the check for the kernel.
+    from oracle.paged_attention_oracle import bf16_bits_to_f32, textbook_prefill_f64
+    exact = np.asarray(textbook_prefill_f64(q, k, v, cu_q, cu_k, c["scale"]), np.float64)
+    err = np.abs(bf16_bits_to_f32(got).astype(np.float64) - exact)
+    assert np.all(err <= 1e-2 + 1e-2 * np.abs(exact)), f"seed={seed}: max err {err.max():.3e} vs float64"
