@@ -249,7 +249,8 @@ def main():
     w = make_workload(args.workload)
     q, kc, vc, bt, ctx, slots, k_new, v_new = device_inputs(w, torch, dev)
     # like the reference's filler, the workload generator knows the lengths on the host
-    chunk = choose_split(w.context_lens, w.num_kv_heads) if args.chunk is None else args.chunk
+    chunk = (choose_split(w.context_lens, w.num_kv_heads, w.num_heads) if args.chunk is None
+             else args.chunk)
     split_name = {0: "balanced", -1: "whole sequence per workgroup"}.get(chunk,
                                                                         f"fixed chunk {chunk}")
     kernel_name = {0: "paged_decode_balanced_kernel", -1: "paged_decode_whole_kernel"}.get(

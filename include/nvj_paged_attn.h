@@ -104,11 +104,13 @@ NVJ_API int32_t nvj_paged_decode_default_chunk(int32_t batch, int32_t num_kv_hea
 
 /*
  * Number of workgroups chunk == NVJ_CHUNK_WHOLE_SEQUENCE launches for a batch:
- * batch * num_kv_heads / (KV heads per workgroup).  One 8-wave workgroup is
+ * batch * num_kv_heads / (KV heads per workgroup; a cache head with more than
+ * 16 query heads counts as several).  One 8-wave workgroup is
  * resident per CU (256 on MI355X), so that mode pays off when this is (just
  * under) a multiple of 256 and the lengths are similar; 0 on invalid arguments.
  */
-NVJ_API int32_t nvj_paged_decode_whole_sequence_workgroups(int32_t batch, int32_t num_kv_heads);
+NVJ_API int32_t nvj_paged_decode_whole_sequence_workgroups(int32_t batch, int32_t num_heads,
+                                                   int32_t num_kv_heads);
 
 /*
  * Bytes of device workspace nvj_paged_decode_launch needs for the partials
@@ -151,8 +153,10 @@ NVJ_API size_t nvj_paged_decode_workspace_bytes(int32_t batch, int32_t num_heads
  * share of positions for all KV heads) and the combine pass; one launch for
  * chunk == NVJ_CHUNK_WHOLE_SEQUENCE.
  * Supported: head_dim 128 (every Qwen3 size) or 64 (the reference's toy test
- * shapes), num_heads / num_kv_heads <= 16, block_size a multiple of 32, chunk
- * a multiple of 32 (0 = balanced split) or NVJ_CHUNK_WHOLE_SEQUENCE.
+ * shapes), block_size a multiple of 32, chunk a multiple of 32 (0 = balanced
+ * split) or NVJ_CHUNK_WHOLE_SEQUENCE.  K/V are read once for up to 16 query
+ * heads per KV head (every Qwen3 size has 2 to 8); a larger group is served in
+ * parts of at most 16, with one read of the KV head's rows per part.
  */
 NVJ_API int nvj_paged_decode_launch(void* stream,
                             const void* q, const void* k_cache, const void* v_cache,

@@ -26,7 +26,7 @@ SYMBOLS = {
         _c.c_void_p, _c.c_void_p, _c.c_void_p, _c.c_void_p, _c.c_void_p, _c.c_void_p,
         _c.c_int32, _c.c_int32, _c.c_int32, _c.c_int64, _c.c_int32, _c.c_int32]),
     "nvj_paged_decode_default_chunk": (_c.c_int32, [_c.c_int32] * 4),
-    "nvj_paged_decode_whole_sequence_workgroups": (_c.c_int32, [_c.c_int32] * 2),
+    "nvj_paged_decode_whole_sequence_workgroups": (_c.c_int32, [_c.c_int32] * 3),
     "nvj_paged_decode_workspace_bytes": (_c.c_size_t, [_c.c_int32] * 7),
     "nvj_paged_decode_launch": (_c.c_int, [
         _c.c_void_p, _c.c_void_p, _c.c_void_p, _c.c_void_p, _c.c_void_p, _c.c_void_p,

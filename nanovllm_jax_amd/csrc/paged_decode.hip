@@ -151,7 +151,11 @@ struct DecodeArgs {
   uint4* out;                  // [B, Hq, 16] pieces (bf16)
   float* part_o;               // [slots, Hq, 128]
   float* part_ml;              // [slots, Hq, 2]
-  int num_heads, num_kv_heads, group, block_size, max_blocks, num_blocks;
+  // num_kv_heads and group describe the heads as the kernels walk them: with
+  // more than 16 query heads per cache head, a cache head is walked as kv_rep
+  // "virtual" KV heads of group = G / kv_rep query heads each (kv_rep = 1
+  // otherwise); cache_kv_heads is the number of heads a cache row really holds.
+  int num_heads, num_kv_heads, group, kv_rep, cache_kv_heads, block_size, max_blocks, num_blocks;
   float scale_log2e;
 };
 
@@ -193,8 +197,8 @@ __device__ __forceinline__ void compute_segment(const DecodeArgs& a, uint4* lds,
     }
   }
 
-  const uint32_t row_bytes = (uint32_t)a.num_kv_heads * (D * 2);  // one position, all heads
-  const int64_t head_bytes = (int64_t)kvh * (D * 2);
+  const uint32_t row_bytes = (uint32_t)a.cache_kv_heads * (D * 2);  // one position, all heads
+  const int64_t head_bytes = (int64_t)(kvh / a.kv_rep) * (D * 2);
   const const_i32_ptr table = as_constant(a.block_tables + (int64_t)b * a.max_blocks);
 
   // wave-uniform byte offset of the first position of a step inside the cache
@@ -673,6 +677,16 @@ __global__ __launch_bounds__(kMaxHeadDim) void paged_decode_combine_kernel(
 
 int round_up(int x, int m) { return (x + m - 1) / m * m; }
 
+// A wave covers at most 16 query heads (the MFMA columns).  A cache head with
+// more than that is walked as `rep` virtual KV heads, the smallest count that
+// divides the group into parts of at most 16; its K/V rows are then read once
+// per virtual head.
+int virtual_heads_per_cache_head(int group) {
+  int rep = 1;
+  while (group % rep != 0 || group / rep > 16) ++rep;
+  return rep;
+}
+
 // Whole-sequence mode: KV heads per 8-wave workgroup.  As many as still give
 // one workgroup per CU (256), so that the split inside a workgroup is no finer
 // than needed; it must divide the number of KV heads.
@@ -750,10 +764,13 @@ extern "C" int32_t nvj_paged_decode_default_chunk(int32_t batch, int32_t num_kv_
   return round_up((int)chunk, kStep);
 }
 
-extern "C" int32_t nvj_paged_decode_whole_sequence_workgroups(int32_t batch,
+extern "C" int32_t nvj_paged_decode_whole_sequence_workgroups(int32_t batch, int32_t num_heads,
                                                                int32_t num_kv_heads) {
-  if (batch <= 0 || num_kv_heads <= 0 || (int64_t)batch * num_kv_heads > INT32_MAX) return 0;
-  return batch * (num_kv_heads / whole_sequence_heads_per_workgroup(batch, num_kv_heads));
+  if (batch <= 0 || num_heads <= 0 || num_kv_heads <= 0 || num_heads % num_kv_heads != 0) return 0;
+  const int64_t heads =
+      (int64_t)num_kv_heads * virtual_heads_per_cache_head(num_heads / num_kv_heads);
+  if (batch * heads > INT32_MAX) return 0;
+  return batch * ((int)heads / whole_sequence_heads_per_workgroup(batch, (int)heads));
 }
 
 extern "C" size_t nvj_paged_decode_workspace_bytes(int32_t batch, int32_t num_heads,
@@ -762,8 +779,10 @@ extern "C" size_t nvj_paged_decode_workspace_bytes(int32_t batch, int32_t num_he
                                                    int32_t chunk) {
   if (chunk == NVJ_CHUNK_WHOLE_SEQUENCE) return 0;   // finished inside the workgroups
   if (batch <= 0 || num_heads <= 0 || (head_dim != 128 && head_dim != 64) || max_blocks <= 0 ||
-      block_size <= 0 || num_kv_heads <= 0 || chunk < 0 || chunk % kStep != 0)
+      block_size <= 0 || num_kv_heads <= 0 || num_heads % num_kv_heads != 0 || chunk < 0 ||
+      chunk % kStep != 0)
     return 0;
+  num_kv_heads *= virtual_heads_per_cache_head(num_heads / num_kv_heads);
   WorkspacePlan plan;
   if (!plan_workspace(batch, num_heads, head_dim, max_blocks, block_size, num_kv_heads, chunk,
                       &plan))
@@ -785,10 +804,14 @@ extern "C" int nvj_paged_decode_launch_phases(void* stream, const void* q, const
       max_blocks < 0 || num_blocks <= 0 || (chunk < 0 && !whole))
     return NVJ_ERR_BAD_SHAPE;
   if (num_heads % num_kv_heads != 0) return NVJ_ERR_BAD_SHAPE;
-  const int group = num_heads / num_kv_heads;
-  if ((head_dim != 128 && head_dim != 64) || group > 16 || block_size % kStep != 0 ||
+  if ((head_dim != 128 && head_dim != 64) || block_size % kStep != 0 ||
       (!whole && chunk % kStep != 0))
     return NVJ_ERR_UNSUPPORTED;
+  const int cache_kv_heads = num_kv_heads;
+  const int kv_rep = virtual_heads_per_cache_head(num_heads / num_kv_heads);
+  if ((int64_t)num_kv_heads * kv_rep > INT32_MAX) return NVJ_ERR_BAD_SHAPE;
+  num_kv_heads *= kv_rep;   // from here on: the heads as the kernels walk them
+  const int group = num_heads / num_kv_heads;
   if ((int64_t)max_blocks * block_size > INT32_MAX) return NVJ_ERR_BAD_SHAPE;
   if (!(scale >= 0.f)) return NVJ_ERR_BAD_SHAPE;   // the running max assumes a non-negative scale
   if (batch == 0) return NVJ_OK;
@@ -812,6 +835,8 @@ extern "C" int nvj_paged_decode_launch_phases(void* stream, const void* q, const
   a.num_heads = num_heads;
   a.num_kv_heads = num_kv_heads;
   a.group = group;
+  a.kv_rep = kv_rep;
+  a.cache_kv_heads = cache_kv_heads;
   a.block_size = block_size;
   a.max_blocks = max_blocks;
   a.num_blocks = num_blocks;

@@ -286,7 +286,7 @@ class DecodeStepRunner:
         d = self.device
         t = lambda a: torch.from_numpy(a).to(d)
         # the lengths are host integers here, as in the reference's filler: pick the split
-        split = choose_split(ctx, self.cfg.num_kv_heads)
+        split = choose_split(ctx, self.cfg.num_kv_heads, self.cfg.num_heads)
         return t(ids), t(pos), create_decode_context(t(ctx), t(slots), t(bt), split)
 
     def make_prefill_inputs(self, token_lists, block_tables):

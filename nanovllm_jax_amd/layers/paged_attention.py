@@ -48,7 +48,7 @@ def paged_decode_workspace_bytes(batch: int, num_heads: int, head_dim: int,
         batch, num_heads, head_dim, max_blocks, block_size, num_kv_heads, chunk))
 
 
-def choose_split(context_lens_host, num_kv_heads: int) -> int:
+def choose_split(context_lens_host, num_kv_heads: int, num_heads: int | None = None) -> int:
     """``chunk`` for a batch whose lengths the host knows (the reference's filler
     builds ``context_lens`` from Python ints, ``engine/model_runner.py:334-376``):
     ``WHOLE_SEQUENCE`` when the longest sequence is within 10 % of the mean and
@@ -60,7 +60,8 @@ def choose_split(context_lens_host, num_kv_heads: int) -> int:
     mean = sum(lens) / len(lens)
     if mean <= 0 or max(lens) > 1.1 * mean:
         return 0
-    wgs = int(_lib.load().nvj_paged_decode_whole_sequence_workgroups(len(lens), num_kv_heads))
+    wgs = int(_lib.load().nvj_paged_decode_whole_sequence_workgroups(
+        len(lens), num_kv_heads if num_heads is None else num_heads, num_kv_heads))
     rounds = -(-wgs // 256)
     return WHOLE_SEQUENCE if wgs > 0 and wgs >= 0.95 * rounds * 256 else 0
 

@@ -47,7 +47,6 @@ def test_argument_validation_without_a_gpu():
 
     assert call(D=96) == -3                # head_dim not built (128 and 64 are)
     assert call(Hq=30) == -2               # Hq % Hkv
-    assert call(Hq=256, Hkv=8) == -3       # group > 16
     assert call(bs=48) == -3
     assert call(chunk=100) == -3
     assert call(chunk=-2) == -2                   # only -1 (whole sequence) is a mode below 0

@@ -350,3 +350,19 @@ def test_scale_zero_gives_the_mean_of_v_over_the_live_positions(chunk):
         rows = np.concatenate([v[bt[b, p]] for p in range(-(-int(ctx[b]) // bs))])[:ctx[b]]
         mean = np.repeat(rows.mean(axis=0), Hq // Hkv, axis=0)          # [Hq, D]
         assert np.all(np.abs(got[b] - mean) <= 1e-2 + 1e-2 * np.abs(mean)), f"sequence {b}"
+
+
+@pytest.mark.parametrize("Hq,Hkv,D", [(32, 1, 128), (48, 2, 128), (17, 1, 128), (64, 2, 64),
+                                      (40, 1, 64)])
+@pytest.mark.parametrize("chunk", [0, 64, -1])
+def test_more_than_16_query_heads_per_kv_head(Hq, Hkv, D, chunk):
+    """Groups above the 16 MFMA columns of a wave are served in parts (32 = 2 x 16,
+    24 = 2 x 12, 17 = 17 x 1, 40 = 4 x 10), every part reading its KV head's rows."""
+    print(f"case large group Hq={Hq} Hkv={Hkv} D={D} chunk={chunk}", flush=True)
+    B, bs, NB = 9, 64, 60
+    ctx = [0, 1, 33, 64, 100, 257, 300, 31, 129]
+    q, kc, vc, bt, ctx = make_problem(600 + Hq + Hkv, B, Hq, Hkv, D, bs, NB, ctx)
+    scale = 1.0 / np.sqrt(D)
+    got = run_hip(q, kc, vc, bt, ctx, scale, bs, chunk)
+    want = oracle(q, kc, vc, bt, ctx, scale, bs)
+    assert_close_bf16(got, want, what=f"large group Hq={Hq} Hkv={Hkv} chunk={chunk}")

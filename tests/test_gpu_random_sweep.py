@@ -11,7 +11,7 @@ pytestmark = pytest.mark.gpu
 
 def _decode_case(rng):
     Hkv = int(rng.choice([1, 2, 3, 4, 5, 6, 7, 8, 12, 16]))
-    G = int(rng.choice([1, 2, 3, 4, 5, 7, 8, 16]))
+    G = int(rng.choice([1, 2, 3, 4, 5, 7, 8, 16, 20, 32]))
     D = int(rng.choice([128, 128, 64]))
     bs = int(rng.choice([32, 64, 96, 160, 256]))
     B = int(rng.choice([1, 2, 7, 33, 65, 130]))
