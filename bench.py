@@ -36,26 +36,28 @@ MEASURED_TRAFFIC_BYTES = {("C2", 0): 1_080_210_000, ("C2", 1024): 1_080_188_000,
                           ("C2", -1): 1_074_909_000}
 
 
-def device_inputs(w, torch, dev):
-    """Seeded N(0,1) bf16 q / K / V drawn on the device, plus the metadata."""
+def device_inputs(w, torch, dev, dt=None):
+    """Seeded N(0,1) q / K / V of dtype `dt` (bf16 by default) drawn on the
+    device, plus the metadata."""
+    dt = dt or torch.bfloat16
     g = torch.Generator(device=dev)
     g.manual_seed(w.seed)
     shape = (w.num_blocks, w.block_size, w.num_kv_heads, w.head_dim)
-    kc = torch.empty(shape, dtype=torch.bfloat16, device=dev)
-    vc = torch.empty(shape, dtype=torch.bfloat16, device=dev)
+    kc = torch.empty(shape, dtype=dt, device=dev)
+    vc = torch.empty(shape, dtype=dt, device=dev)
     # page by page keeps the fp32 temporaries small at the multi-GiB configs
     step = max(1, (1 << 26) // (w.block_size * w.num_kv_heads * w.head_dim))
     for t in (kc, vc):
         for p0 in range(0, w.num_blocks, step):
             n = min(step, w.num_blocks - p0)
             t[p0:p0 + n] = torch.randn((n,) + shape[1:], generator=g, device=dev,
-                                       dtype=torch.float32).to(torch.bfloat16)
+                                       dtype=torch.float32).to(dt)
     q = (torch.randn((w.batch, w.num_heads, w.head_dim), generator=g, device=dev,
-                     dtype=torch.float32) * w.q_gain).to(torch.bfloat16)
+                     dtype=torch.float32) * w.q_gain).to(dt)
     k_new = torch.randn((w.batch, w.num_kv_heads, w.head_dim), generator=g, device=dev,
                         dtype=torch.float32)
     v_new = torch.randn((w.batch, w.num_kv_heads, w.head_dim), generator=g, device=dev,
-                        dtype=torch.float32).to(torch.bfloat16)
+                        dtype=torch.float32).to(dt)
     bt = torch.from_numpy(w.block_tables).to(dev)
     ctx = torch.from_numpy(w.context_lens).to(dev)
     slots = torch.from_numpy(w.slot_mapping).to(dev)
@@ -211,6 +213,9 @@ def main():
                     help="split mode: 0 = balanced, > 0 = positions per workgroup, -1 = whole "
                          "sequence per workgroup; default: what the host filler would pick from "
                          "the workload's lengths (layers.paged_attention.choose_split)")
+    ap.add_argument("--dtype", default="bf16", choices=["bf16", "f16"],
+                    help="cache / q / out dtype; f16 is what the reference's own timing "
+                         "scripts use (no CPU baseline leg: the C restatement reads bf16)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run a plain 1 GiB device-to-device copy a few times, so a "
@@ -247,7 +252,8 @@ def main():
     if args.prefill:
         return bench_prefill(args, torch)
     w = make_workload(args.workload)
-    q, kc, vc, bt, ctx, slots, k_new, v_new = device_inputs(w, torch, dev)
+    dt = torch.float16 if args.dtype == "f16" else torch.bfloat16
+    q, kc, vc, bt, ctx, slots, k_new, v_new = device_inputs(w, torch, dev, dt)
     # like the reference's filler, the workload generator knows the lengths on the host
     chunk = (choose_split(w.context_lens, w.num_kv_heads, w.num_heads) if args.chunk is None
              else args.chunk)
@@ -294,7 +300,7 @@ def main():
                   if w.name == "C2" else f"paged decode attn HBM GB/s, workload {w.name}",
         "value": round(gbps, 1), "unit": "GB/s", "n_gpus": 1, "steps": args.steps,
         "warmup": args.warmup, "ms_per_step": round(ms_wall, 5), "higher_is_better": True,
-        "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
+        "scaling": "weak", "vs_baseline": None, "dtype": args.dtype, "data": "synthetic",
         "us_per_call": round(ms_call * 1e3, 2),
         "pct_of_hbm_peak": round(100.0 * gbps / HBM_PEAK_GBPS, 2),
         "config": {"workload": f"{w.name}: B={w.batch} Hq={w.num_heads} Hkv={w.num_kv_heads} "
@@ -314,7 +320,7 @@ def main():
                                  None if chunk == -1 else round(ms_combine * 1e3, 2),
                                  "store_kvcache_kernel": round(ms_store * 1e3, 2)},
     }
-    if not args.no_cpu_baseline:
+    if not args.no_cpu_baseline and args.dtype == "bf16":
         rec["cpu_baseline"] = cpu_baseline(w, q, kc, vc, args.cpu_budget)
     print(json.dumps(rec), flush=True)
     return 0

@@ -34,11 +34,13 @@ extern "C" {
 #define NVJ_ERR_LAUNCH        -5   /* hipGetLastError() != hipSuccess after launch  */
 #define NVJ_ERR_BAD_DTYPE     -6   /* unknown element type code                     */
 
-/* element type codes for the new K/V rows handed to the store */
 #define NVJ_CHUNK_WHOLE_SEQUENCE (-1)   /* see the split modes of the paged decode */
 
+/* element type codes: the cache (and q / out) is bf16 or IEEE half; float32 is
+ * accepted only for the new K/V rows handed to the store */
 #define NVJ_DTYPE_BF16 0
 #define NVJ_DTYPE_F32  1
+#define NVJ_DTYPE_F16  2
 
 /* Human-readable text for an NVJ_ERR_* code (static storage). */
 NVJ_API const char* nvj_error_string(int code);
@@ -51,14 +53,15 @@ NVJ_API int nvj_abi_version(void);
  * called from Attention.__call__ on the flattened cache
  * (layers/attention.py:457-475).
  *
- *   key   [num_tokens, num_kv_heads, head_dim]  k_dtype (bf16 or f32; the
+ *   key   [num_tokens, num_kv_heads, head_dim]  k_dtype: cache_dtype, or f32 (the
  *         reference hands over f32 keys after RoPE and casts, :70)
- *   value [num_tokens, num_kv_heads, head_dim]  v_dtype
- *   k_cache, v_cache [num_slots, num_kv_heads, head_dim] bf16, updated IN PLACE
- *         (num_slots = num_blocks * block_size)
+ *   value [num_tokens, num_kv_heads, head_dim]  v_dtype: cache_dtype or f32
+ *   k_cache, v_cache [num_slots, num_kv_heads, head_dim] cache_dtype (bf16 or
+ *         f16, the model dtype of the reference, engine/model_runner.py:176),
+ *         updated IN PLACE (num_slots = num_blocks * block_size)
  *   slot_mapping [num_tokens] int32
  *
- * cache[slot[i]] = bf16_round_nearest_even(x[i]) for 0 <= slot[i] < num_slots;
+ * cache[slot[i]] = round_nearest_even_to_cache_dtype(x[i]) for 0 <= slot[i] < num_slots;
  * slot[i] >= num_slots is dropped (mode='drop', :74); slot[i] < 0 is SKIPPED
  * (the documented meaning of -1, :57-58 -- the reference's code would write
  * row 0 instead).  Rows not named by slot_mapping are not touched.  Duplicate
@@ -71,7 +74,7 @@ NVJ_API int nvj_store_kvcache_launch(void* stream,
                              const int32_t* slot_mapping,
                              int32_t num_tokens, int32_t num_kv_heads,
                              int32_t head_dim, int64_t num_slots,
-                             int32_t k_dtype, int32_t v_dtype);
+                             int32_t k_dtype, int32_t v_dtype, int32_t cache_dtype);
 
 /*
  * How the positions of a call are split over workgroups is chosen by `chunk`:
@@ -131,19 +134,21 @@ NVJ_API size_t nvj_paged_decode_workspace_bytes(int32_t batch, int32_t num_heads
  * Attention._decode_attention (layers/attention.py:389-397), and equally the
  * gather + dot_product_attention fallback (layers/attention.py:399-434).
  *
- *   q            [batch, num_heads, head_dim]                         bf16
- *   k_cache, v_cache [num_blocks, block_size, num_kv_heads, head_dim] bf16
+ *   q            [batch, num_heads, head_dim]                         dtype
+ *   k_cache, v_cache [num_blocks, block_size, num_kv_heads, head_dim] dtype
  *   block_tables [batch, max_blocks] int32; entries at or beyond
  *                ceil(context_lens[b] / block_size) are never read (the
  *                reference pads them with -1, engine/model_runner.py:240)
  *   context_lens [batch] int32 (counts the position being decoded,
  *                engine/model_runner.py:360)
- *   out          [batch, num_heads, head_dim]                         bf16
+ *   out          [batch, num_heads, head_dim]                         dtype
  *   workspace    >= nvj_paged_decode_workspace_bytes(...) bytes, 16-byte aligned,
  *                contents need not be initialised
  *
  * out[b,h,:] = softmax_{s < ctx[b]}(scale * q[b,h,:] . K[b,s,h/G,:]) V[b,s,h/G,:]
- * with G = num_heads / num_kv_heads, fp32 accumulation, bf16 result.
+ * with G = num_heads / num_kv_heads, fp32 accumulation, result in `dtype`
+ * (NVJ_DTYPE_BF16 or NVJ_DTYPE_F16: the cache dtype of the reference is its model
+ * dtype, and its own timing scripts use float16).
  * context_lens[b] <= 0 gives a row of zeros (0 / (0 + 1e-9), :227).  Positions
  * >= context_lens[b] are never read.  Table entries of live pages must lie in
  * [0, num_blocks); the kernel clamps them into range like the reference (:185)
@@ -164,7 +169,7 @@ NVJ_API int nvj_paged_decode_launch(void* stream,
                             void* out, void* workspace, size_t workspace_bytes,
                             int32_t batch, int32_t num_heads, int32_t num_kv_heads,
                             int32_t head_dim, int32_t block_size, int32_t max_blocks,
-                            int32_t num_blocks, float scale, int32_t chunk);
+                            int32_t num_blocks, float scale, int32_t chunk, int32_t dtype);
 
 /*
  * The same call with its two launches selectable: NVJ_PHASE_SPLITK runs the
@@ -182,7 +187,7 @@ NVJ_API int nvj_paged_decode_launch_phases(void* stream,
                             void* out, void* workspace, size_t workspace_bytes,
                             int32_t batch, int32_t num_heads, int32_t num_kv_heads,
                             int32_t head_dim, int32_t block_size, int32_t max_blocks,
-                            int32_t num_blocks, float scale, int32_t chunk,
+                            int32_t num_blocks, float scale, int32_t chunk, int32_t dtype,
                             uint32_t phases);
 
 /*

@@ -16,6 +16,7 @@ _LIB_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), "_native",
 NVJ_ABI_VERSION = 1
 NVJ_DTYPE_BF16 = 0
 NVJ_DTYPE_F32 = 1
+NVJ_DTYPE_F16 = 2
 
 # every symbol include/nvj_paged_attn.h declares: name -> (restype, argtypes)
 _c = ctypes
@@ -24,7 +25,7 @@ SYMBOLS = {
     "nvj_abi_version": (_c.c_int, []),
     "nvj_store_kvcache_launch": (_c.c_int, [
         _c.c_void_p, _c.c_void_p, _c.c_void_p, _c.c_void_p, _c.c_void_p, _c.c_void_p,
-        _c.c_int32, _c.c_int32, _c.c_int32, _c.c_int64, _c.c_int32, _c.c_int32]),
+        _c.c_int32, _c.c_int32, _c.c_int32, _c.c_int64, _c.c_int32, _c.c_int32, _c.c_int32]),
     "nvj_paged_decode_default_chunk": (_c.c_int32, [_c.c_int32] * 4),
     "nvj_paged_decode_whole_sequence_workgroups": (_c.c_int32, [_c.c_int32] * 3),
     "nvj_paged_decode_workspace_bytes": (_c.c_size_t, [_c.c_int32] * 7),
@@ -32,12 +33,12 @@ SYMBOLS = {
         _c.c_void_p, _c.c_void_p, _c.c_void_p, _c.c_void_p, _c.c_void_p, _c.c_void_p,
         _c.c_void_p, _c.c_void_p, _c.c_size_t,
         _c.c_int32, _c.c_int32, _c.c_int32, _c.c_int32, _c.c_int32, _c.c_int32,
-        _c.c_int32, _c.c_float, _c.c_int32]),
+        _c.c_int32, _c.c_float, _c.c_int32, _c.c_int32]),
     "nvj_paged_decode_launch_phases": (_c.c_int, [
         _c.c_void_p, _c.c_void_p, _c.c_void_p, _c.c_void_p, _c.c_void_p, _c.c_void_p,
         _c.c_void_p, _c.c_void_p, _c.c_size_t,
         _c.c_int32, _c.c_int32, _c.c_int32, _c.c_int32, _c.c_int32, _c.c_int32,
-        _c.c_int32, _c.c_float, _c.c_int32, _c.c_uint32]),
+        _c.c_int32, _c.c_float, _c.c_int32, _c.c_int32, _c.c_uint32]),
     "nvj_qk_norm_rope_store_launch": (_c.c_int, [
         _c.c_void_p, _c.c_void_p, _c.c_int64, _c.c_void_p, _c.c_void_p, _c.c_int32, _c.c_void_p,
         _c.c_void_p, _c.c_float, _c.c_void_p, _c.c_void_p, _c.c_void_p, _c.c_void_p,

@@ -58,13 +58,35 @@ template <int D> struct HeadDim {
 constexpr float kNegBig = -1.0e30f;  // stands for -inf without inf-inf hazards
 constexpr float kLog2e = 1.4426950408889634f;
 
-__device__ __forceinline__ bf16x8 as_bf16x8(uint4 v) { return __builtin_bit_cast(bf16x8, v); }
+typedef __attribute__((ext_vector_type(8))) _Float16 f16x8;
 
-__device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi) {
-  typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2;
-  bf16x2 p = {(__bf16)lo, (__bf16)hi};
-  return __builtin_bit_cast(uint32_t, p);
-}
+// The cache element type: bf16 (F16 = false) or IEEE half (F16 = true).  The
+// kernels move 16-bit patterns; only the matrix instruction, the rounding of
+// the probabilities and of the output depend on the type.
+template <bool F16> struct Elem;
+template <> struct Elem<false> {
+  static __device__ __forceinline__ f32x4 mfma(uint4 a, uint4 b, f32x4 c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a),
+                                                   __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
+  }
+  static __device__ __forceinline__ uint32_t pack2(float lo, float hi) {
+    typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2;
+    bf16x2 p = {(__bf16)lo, (__bf16)hi};
+    return __builtin_bit_cast(uint32_t, p);
+  }
+};
+template <> struct Elem<true> {
+  static __device__ __forceinline__ f32x4 mfma(uint4 a, uint4 b, f32x4 c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8, a),
+                                                  __builtin_bit_cast(f16x8, b), c, 0, 0, 0);
+  }
+  static __device__ __forceinline__ uint32_t pack2(float lo, float hi) {
+    typedef __attribute__((ext_vector_type(2))) _Float16 f16x2;
+    f16x2 p = {(_Float16)lo, (_Float16)hi};   // round to nearest even
+    return __builtin_bit_cast(uint32_t, p);
+  }
+};
+
 
 __device__ __forceinline__ float wave_xor_max(float x, int mask) {
   return fmaxf(x, __shfl_xor(x, mask, 64));
@@ -165,7 +187,7 @@ struct DecodeArgs {
 // lane (r = lane & 15, kg = lane >> 4), m_run the maximum raw score and l_run
 // the sum of exp((score - m_run) * scale) of that head (the same in the four
 // lanes that share r).  Lanes with r >= group hold padding.
-template <int D>
+template <int D, bool F16>
 __device__ __forceinline__ void compute_segment(const DecodeArgs& a, uint4* lds, int b, int kvh,
                                                 int t0, int t1, int lane, f32x4 (&acc)[8],
                                                 float& m_run, float& l_run) {
@@ -183,7 +205,7 @@ __device__ __forceinline__ void compute_segment(const DecodeArgs& a, uint4* lds,
   // Q^T as MFMA B operand for the D/32 reduction steps over head_dim:
   // lane (column r = query head of the group, k-group kg) holds dims
   // 32*s + 8*kg .. +8.  Columns >= group are zero.
-  bf16x8 qreg[H::kQkSteps];
+  uint4 qreg[H::kQkSteps];
   {
     // lanes of padding columns read the group's last head (always in range)
     // and then drop it, so the loads stay unconditional 16-byte loads
@@ -193,7 +215,7 @@ __device__ __forceinline__ void compute_segment(const DecodeArgs& a, uint4* lds,
 #pragma unroll
     for (int s = 0; s < H::kQkSteps; ++s) {
       const uint4 v = qrow[4 * s + kg];
-      qreg[s] = as_bf16x8(r < group ? v : zero);
+      qreg[s] = r < group ? v : zero;
     }
   }
 
@@ -248,10 +270,10 @@ __device__ __forceinline__ void compute_segment(const DecodeArgs& a, uint4* lds,
     f32x4 s0 = {0.f, 0.f, 0.f, 0.f}, s1 = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
     for (int s = 0; s < H::kQkSteps; ++s) {
-      const bf16x8 a0 = as_bf16x8(lds[r * H::kLdsRowPieces + 4 * s + kg]);
-      const bf16x8 a1 = as_bf16x8(lds[(16 + r) * H::kLdsRowPieces + 4 * s + kg]);
-      s0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a0, qreg[s], s0, 0, 0, 0);
-      s1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a1, qreg[s], s1, 0, 0, 0);
+      const uint4 a0 = lds[r * H::kLdsRowPieces + 4 * s + kg];
+      const uint4 a1 = lds[(16 + r) * H::kLdsRowPieces + 4 * s + kg];
+      s0 = Elem<F16>::mfma(a0, qreg[s], s0);
+      s1 = Elem<F16>::mfma(a1, qreg[s], s1);
     }
 
     // ---- online softmax; lane holds positions 4*kg+e (s0) and 16+4*kg+e (s1) ----
@@ -290,11 +312,10 @@ __device__ __forceinline__ void compute_segment(const DecodeArgs& a, uint4* lds,
     for (int e = 0; e < 4; ++e) psum += p0[e] + p1[e];
     l_run = fmaf(l_run, alpha, psum);
     uint4 pbits;
-    pbits.x = pack_bf16x2(p0[0], p0[1]);
-    pbits.y = pack_bf16x2(p0[2], p0[3]);
-    pbits.z = pack_bf16x2(p1[0], p1[1]);
-    pbits.w = pack_bf16x2(p1[2], p1[3]);
-    const bf16x8 pb = as_bf16x8(pbits);
+    pbits.x = Elem<F16>::pack2(p0[0], p0[1]);
+    pbits.y = Elem<F16>::pack2(p0[2], p0[3]);
+    pbits.z = Elem<F16>::pack2(p1[0], p1[1]);
+    pbits.w = Elem<F16>::pack2(p1[2], p1[3]);
 
     // ---- V: in-lane 8x8 transpose (positions x dims), then next V loads ----
     uint4 vt[8];
@@ -325,7 +346,7 @@ __device__ __forceinline__ void compute_segment(const DecodeArgs& a, uint4* lds,
 #pragma unroll
     for (int jd = 0; jd < 8; ++jd) {
       acc[jd] *= alpha;
-      acc[jd] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(vt[jd]), pb, acc[jd], 0, 0, 0);
+      acc[jd] = Elem<F16>::mfma(vt[jd], pbits, acc[jd]);
     }
   }
 
@@ -335,7 +356,7 @@ __device__ __forceinline__ void compute_segment(const DecodeArgs& a, uint4* lds,
 }
 
 // Normalised bf16 result of a whole sequence straight to `out`.
-template <int D>
+template <int D, bool F16>
 __device__ __forceinline__ void write_output(const DecodeArgs& a, int b, int kvh, int lane,
                                              const f32x4 (&acc)[8], float l_run) {
   using H = HeadDim<D>;
@@ -348,10 +369,10 @@ __device__ __forceinline__ void write_output(const DecodeArgs& a, int b, int kvh
 #pragma unroll
   for (int e = 0; e < 4; ++e) {
     uint4 o;
-    o.x = pack_bf16x2(acc[0][e] * inv, acc[1][e] * inv);
-    o.y = pack_bf16x2(acc[2][e] * inv, acc[3][e] * inv);
-    o.z = pack_bf16x2(acc[4][e] * inv, acc[5][e] * inv);
-    o.w = pack_bf16x2(acc[6][e] * inv, acc[7][e] * inv);
+    o.x = Elem<F16>::pack2(acc[0][e] * inv, acc[1][e] * inv);
+    o.y = Elem<F16>::pack2(acc[2][e] * inv, acc[3][e] * inv);
+    o.z = Elem<F16>::pack2(acc[4][e] * inv, acc[5][e] * inv);
+    o.w = Elem<F16>::pack2(acc[6][e] * inv, acc[7][e] * inv);
     orow[e] = o;
   }
 }
@@ -374,21 +395,21 @@ __device__ __forceinline__ void write_partial(const DecodeArgs& a, int64_t slot,
 
 // compute_segment, then: `direct` (the segment is the whole sequence) -> out,
 // otherwise -> partial slot `slot`.
-template <int D>
+template <int D, bool F16>
 __device__ __forceinline__ void run_segment(const DecodeArgs& a, uint4* lds, int b, int kvh,
                                             int t0, int t1, int64_t slot, bool direct,
                                             int lane) {
   f32x4 acc[8];
   float m_run, l_run;
-  compute_segment<D>(a, lds, b, kvh, t0, t1, lane, acc, m_run, l_run);
-  if (direct) write_output<D>(a, b, kvh, lane, acc, l_run);
+  compute_segment<D, F16>(a, lds, b, kvh, t0, t1, lane, acc, m_run, l_run);
+  if (direct) write_output<D, F16>(a, b, kvh, lane, acc, l_run);
   else write_partial<D>(a, slot, kvh, lane, acc, m_run, l_run);
 }
 
 // Fixed-chunk split: grid.x = batch * max_chunks, grid.y = num_kv_heads / NW,
 // block = NW * 64.  Workgroup (b, c) owns positions [c*chunk, (c+1)*chunk) of
 // sequence b; partial slot = b * max_chunks + c.
-template <int NW, int D>
+template <int NW, int D, bool F16>
 __global__ __launch_bounds__(NW * 64) void paged_decode_splitk_kernel(DecodeArgs a, int chunk,
                                                                       int max_chunks) {
   __shared__ uint4 k_tile[NW][kStep * HeadDim<D>::kLdsRowPieces];
@@ -402,8 +423,8 @@ __global__ __launch_bounds__(NW * 64) void paged_decode_splitk_kernel(DecodeArgs
   if (t0 >= ctx) return;  // also every chunk of an empty sequence
   const int t1 = min(ctx, t0 + chunk);
   const bool direct = ctx <= chunk;
-  run_segment<D>(a, k_tile[wave], b, blockIdx.y * NW + wave, t0, t1,
-                 (int64_t)b * max_chunks + c, direct, lane);
+  run_segment<D, F16>(a, k_tile[wave], b, blockIdx.y * NW + wave, t0, t1,
+                      (int64_t)b * max_chunks + c, direct, lane);
 }
 
 // Whole-sequence split: every sequence is finished inside one workgroup, so
@@ -415,7 +436,7 @@ __global__ __launch_bounds__(NW * 64) void paged_decode_splitk_kernel(DecodeArgs
 // wave's K tile is free by then and exactly holds its 34 floats per lane) and
 // the wave of part 0 merges them and writes the output.  Meant for batches of
 // similar lengths: a workgroup's time follows its sequence's length.
-template <int NW, int D>
+template <int NW, int D, bool F16>
 __global__ __launch_bounds__(NW * 64) void paged_decode_whole_kernel(DecodeArgs a, int hpw) {
   using H = HeadDim<D>;
   __shared__ uint4 k_tile[NW][kStep * H::kLdsRowPieces];
@@ -440,8 +461,8 @@ __global__ __launch_bounds__(NW * 64) void paged_decode_whole_kernel(DecodeArgs 
   for (int jd = 0; jd < 8; ++jd) acc[jd] = f32x4{0.f, 0.f, 0.f, 0.f};
   float m_run = kNegBig, l_run = 0.f;
   if (s1 > s0)
-    compute_segment<D>(a, k_tile[wave], b, kvh, s0 * kStep, min(ctx, s1 * kStep), lane, acc, m_run,
-                       l_run);
+    compute_segment<D, F16>(a, k_tile[wave], b, kvh, s0 * kStep, min(ctx, s1 * kStep), lane, acc,
+                            m_run, l_run);
   if (parts > 1) {
     // value v of lane l at float v * kLanesWithDims + l of the wave's tile
     const bool holds_dims = lane < kLanesWithDims;
@@ -474,7 +495,7 @@ __global__ __launch_bounds__(NW * 64) void paged_decode_whole_kernel(DecodeArgs 
       }
     }
   }
-  write_output<D>(a, b, kvh, lane, acc, l_run);
+  write_output<D, F16>(a, b, kvh, lane, acc, l_run);
 }
 
 // Inclusive prefix sum over the 64 lanes of a wave with DPP moves: a
@@ -502,7 +523,7 @@ __device__ __forceinline__ int wave_inclusive_scan(int x) {
 // never needs the lengths.  Workgroup 0 also leaves the exclusive prefix sums
 // (steps before each sequence, total at [batch]) in `prefix` for the combine
 // pass.  grid.x = num_wgs, grid.y = num_kv_heads / NW, block = NW * 64.
-template <int NW, int D>
+template <int NW, int D, bool F16>
 __global__ __launch_bounds__(NW * 64) void paged_decode_balanced_kernel(DecodeArgs a, int batch,
                                                                         int num_wgs,
                                                                         int min_steps,
@@ -607,8 +628,8 @@ __global__ __launch_bounds__(NW * 64) void paged_decode_balanced_kernel(DecodeAr
     const int t0 = __builtin_amdgcn_readfirstlane((pos - before) * kStep);
     const int t1 = __builtin_amdgcn_readfirstlane(min(ctx, (seg_end - before) * kStep));
     const bool direct = pos == before && seg_end == before + nb;
-    run_segment<D>(a, k_tile[wave], sb, blockIdx.y * NW + wave, t0, t1, (int64_t)(g + sb),
-                   direct, lane);
+    run_segment<D, F16>(a, k_tile[wave], sb, blockIdx.y * NW + wave, t0, t1, (int64_t)(g + sb),
+                        direct, lane);
     pos = seg_end;
   }
 }
@@ -623,7 +644,7 @@ __global__ __launch_bounds__(kMaxHeadDim) void paged_decode_combine_kernel(
     const float* __restrict__ part_o, const float* __restrict__ part_ml,
     const int32_t* __restrict__ context_lens, const int32_t* __restrict__ prefix,
     uint16_t* __restrict__ out, int num_heads, int chunk, int max_chunks, int max_positions,
-    int batch, int num_wgs, int min_steps, float scale_log2e) {
+    int batch, int num_wgs, int min_steps, float scale_log2e, bool f16) {
   const int b = blockIdx.x, h = blockIdx.y, d = threadIdx.x;
   const int head_dim = blockDim.x;
   int nparts;
@@ -672,7 +693,7 @@ __global__ __launch_bounds__(kMaxHeadDim) void paged_decode_combine_kernel(
     }
   }
   const float res = num / (den + 1e-9f);
-  *o = (uint16_t)(pack_bf16x2(res, 0.f) & 0xFFFFu);
+  *o = (uint16_t)((f16 ? Elem<true>::pack2(res, 0.f) : Elem<false>::pack2(res, 0.f)) & 0xFFFFu);
 }
 
 int round_up(int x, int m) { return (x + m - 1) / m * m; }
@@ -798,7 +819,9 @@ extern "C" int nvj_paged_decode_launch_phases(void* stream, const void* q, const
                                               int32_t num_kv_heads, int32_t head_dim,
                                               int32_t block_size, int32_t max_blocks,
                                               int32_t num_blocks, float scale, int32_t chunk,
-                                              uint32_t phases) {
+                                              int32_t dtype, uint32_t phases) {
+  if (dtype != NVJ_DTYPE_BF16 && dtype != NVJ_DTYPE_F16) return NVJ_ERR_BAD_DTYPE;
+  const bool f16 = dtype == NVJ_DTYPE_F16;
   const bool whole = chunk == NVJ_CHUNK_WHOLE_SEQUENCE;
   if (batch < 0 || num_heads <= 0 || num_kv_heads <= 0 || head_dim <= 0 || block_size <= 0 ||
       max_blocks < 0 || num_blocks <= 0 || (chunk < 0 && !whole))
@@ -847,8 +870,10 @@ extern "C" int nvj_paged_decode_launch_phases(void* stream, const void* q, const
     if (!(phases & NVJ_PHASE_SPLITK)) return NVJ_OK;   // there is no second pass
     const int hpw = whole_sequence_heads_per_workgroup(batch, num_kv_heads);
     const dim3 grid((unsigned)(batch * (num_kv_heads / hpw)));
-    if (head_dim == 128) paged_decode_whole_kernel<8, 128><<<grid, dim3(512), 0, s>>>(a, hpw);
-    else paged_decode_whole_kernel<8, 64><<<grid, dim3(512), 0, s>>>(a, hpw);
+    if (head_dim == 128 && !f16) paged_decode_whole_kernel<8, 128, false><<<grid, dim3(512), 0, s>>>(a, hpw);
+    else if (head_dim == 128) paged_decode_whole_kernel<8, 128, true><<<grid, dim3(512), 0, s>>>(a, hpw);
+    else if (!f16) paged_decode_whole_kernel<8, 64, false><<<grid, dim3(512), 0, s>>>(a, hpw);
+    else paged_decode_whole_kernel<8, 64, true><<<grid, dim3(512), 0, s>>>(a, hpw);
     return hipGetLastError() == hipSuccess ? NVJ_OK : NVJ_ERR_LAUNCH;
   }
 
@@ -867,33 +892,39 @@ extern "C" int nvj_paged_decode_launch_phases(void* stream, const void* q, const
       const int nw = waves_per_workgroup(num_kv_heads);
       const unsigned gy = (unsigned)(num_kv_heads / nw);
       // one instantiation per (waves per workgroup, head_dim)
-#define NVJ_FOR_SHAPE(LAUNCH)                 \
-  switch (nw * 1000 + head_dim) {             \
-    case 8128: LAUNCH(8, 128); break;         \
-    case 4128: LAUNCH(4, 128); break;         \
-    case 2128: LAUNCH(2, 128); break;         \
-    case 1128: LAUNCH(1, 128); break;         \
-    case 8064: LAUNCH(8, 64); break;          \
-    case 4064: LAUNCH(4, 64); break;          \
-    case 2064: LAUNCH(2, 64); break;          \
-    default: LAUNCH(1, 64); break;            \
+#define NVJ_FOR_DTYPE(LAUNCH, NWV, DV) \
+  do {                                \
+    if (f16) LAUNCH(NWV, DV, true);   \
+    else LAUNCH(NWV, DV, false);      \
+  } while (0)
+#define NVJ_FOR_SHAPE(LAUNCH)                             \
+  switch (nw * 1000 + head_dim) {                         \
+    case 8128: NVJ_FOR_DTYPE(LAUNCH, 8, 128); break;      \
+    case 4128: NVJ_FOR_DTYPE(LAUNCH, 4, 128); break;      \
+    case 2128: NVJ_FOR_DTYPE(LAUNCH, 2, 128); break;      \
+    case 1128: NVJ_FOR_DTYPE(LAUNCH, 1, 128); break;      \
+    case 8064: NVJ_FOR_DTYPE(LAUNCH, 8, 64); break;       \
+    case 4064: NVJ_FOR_DTYPE(LAUNCH, 4, 64); break;       \
+    case 2064: NVJ_FOR_DTYPE(LAUNCH, 2, 64); break;       \
+    default: NVJ_FOR_DTYPE(LAUNCH, 1, 64); break;         \
   }
       if (chunk == 0) {
         const dim3 grid((unsigned)plan.num_wgs, gy);
-#define NVJ_LAUNCH_BALANCED(NWV, DV)                                      \
-  paged_decode_balanced_kernel<NWV, DV><<<grid, dim3(NWV * 64), 0, s>>>( \
+#define NVJ_LAUNCH_BALANCED(NWV, DV, F16V)                                      \
+  paged_decode_balanced_kernel<NWV, DV, F16V><<<grid, dim3(NWV * 64), 0, s>>>( \
       a, batch, plan.num_wgs, kMinBalancedSteps, prefix)
         NVJ_FOR_SHAPE(NVJ_LAUNCH_BALANCED)
 #undef NVJ_LAUNCH_BALANCED
       } else {
         const dim3 grid((unsigned)(batch * plan.max_chunks), gy);
-#define NVJ_LAUNCH_FIXED(NWV, DV)                                                    \
-  paged_decode_splitk_kernel<NWV, DV><<<grid, dim3(NWV * 64), 0, s>>>(a, chunk, \
-                                                                       plan.max_chunks)
+#define NVJ_LAUNCH_FIXED(NWV, DV, F16V)                                                    \
+  paged_decode_splitk_kernel<NWV, DV, F16V><<<grid, dim3(NWV * 64), 0, s>>>(a, chunk, \
+                                                                             plan.max_chunks)
         NVJ_FOR_SHAPE(NVJ_LAUNCH_FIXED)
 #undef NVJ_LAUNCH_FIXED
       }
 #undef NVJ_FOR_SHAPE
+#undef NVJ_FOR_DTYPE
       if (hipGetLastError() != hipSuccess) return NVJ_ERR_LAUNCH;
     }
   } else {
@@ -903,7 +934,7 @@ extern "C" int nvj_paged_decode_launch_phases(void* stream, const void* q, const
   paged_decode_combine_kernel<<<dim3((unsigned)batch, (unsigned)num_heads), dim3(head_dim), 0, s>>>(
       a.part_o, a.part_ml, context_lens, prefix, static_cast<uint16_t*>(out), num_heads, chunk,
       plan.max_chunks, max_blocks * block_size, batch, plan.num_wgs, kMinBalancedSteps,
-      a.scale_log2e);
+      a.scale_log2e, f16);
   return hipGetLastError() == hipSuccess ? NVJ_OK : NVJ_ERR_LAUNCH;
 }
 
@@ -913,11 +944,12 @@ extern "C" int nvj_paged_decode_launch(void* stream, const void* q, const void* 
                                        size_t workspace_bytes, int32_t batch, int32_t num_heads,
                                        int32_t num_kv_heads, int32_t head_dim,
                                        int32_t block_size, int32_t max_blocks,
-                                       int32_t num_blocks, float scale, int32_t chunk) {
+                                       int32_t num_blocks, float scale, int32_t chunk,
+                                       int32_t dtype) {
   return nvj_paged_decode_launch_phases(stream, q, k_cache, v_cache, block_tables, context_lens,
                                         out, workspace, workspace_bytes, batch, num_heads,
                                         num_kv_heads, head_dim, block_size, max_blocks,
-                                        num_blocks, scale, chunk,
+                                        num_blocks, scale, chunk, dtype,
                                         NVJ_PHASE_SPLITK | NVJ_PHASE_COMBINE);
 }
 

@@ -5,8 +5,9 @@
 // reference): cast to the cache dtype (:70-71), then cache[slot] = row for
 // every in-range slot (:74-75).  Out-of-range slots are dropped, negative
 // slots are skipped.  HBM-bound byte shuffling: every lane moves one 16-byte
-// piece of a row (8 bf16), reading either 16 bytes (bf16 source) or 32 bytes
-// (f32 source, rounded to nearest even here).
+// piece of a row (8 cache elements, bf16 or IEEE half), reading either 16
+// bytes (source already in the cache's type) or 32 bytes (f32 source, rounded
+// to nearest even here).
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
@@ -22,25 +23,35 @@ __device__ __forceinline__ uint32_t f32_to_bf16_rne(uint32_t u) {
   return is_nan ? ((u >> 16) | 0x0040u) : r;
 }
 
-template <bool F32>
-__device__ __forceinline__ uint4 load_piece_as_bf16(const void* src, int64_t piece) {
+// fp32 -> IEEE half bits, round to nearest even (the hardware conversion).
+__device__ __forceinline__ uint32_t f32_to_f16_rne(uint32_t u) {
+  const _Float16 h = (_Float16)__uint_as_float(u);
+  return (uint32_t)__builtin_bit_cast(uint16_t, h);
+}
+
+// One piece of a source row as 8 cache elements.  F32: the source is float32
+// and is rounded to the cache's type (CF16: IEEE half, else bf16); otherwise
+// the source already has the cache's type and is copied.
+template <bool F32, bool CF16>
+__device__ __forceinline__ uint4 load_piece_as_cache_type(const void* src, int64_t piece) {
   if constexpr (!F32) {
     return reinterpret_cast<const uint4*>(src)[piece];
   } else {
     const uint4* p = reinterpret_cast<const uint4*>(src) + 2 * piece;
     const uint4 a = p[0], b = p[1];
+    auto cvt = [](uint32_t u) { return CF16 ? f32_to_f16_rne(u) : f32_to_bf16_rne(u); };
     uint4 o;
-    o.x = f32_to_bf16_rne(a.x) | (f32_to_bf16_rne(a.y) << 16);
-    o.y = f32_to_bf16_rne(a.z) | (f32_to_bf16_rne(a.w) << 16);
-    o.z = f32_to_bf16_rne(b.x) | (f32_to_bf16_rne(b.y) << 16);
-    o.w = f32_to_bf16_rne(b.z) | (f32_to_bf16_rne(b.w) << 16);
+    o.x = cvt(a.x) | (cvt(a.y) << 16);
+    o.y = cvt(a.z) | (cvt(a.w) << 16);
+    o.z = cvt(b.x) | (cvt(b.y) << 16);
+    o.w = cvt(b.z) | (cvt(b.w) << 16);
     return o;
   }
 }
 
 // One lane per 16-byte piece of one token row, for K and V both.
 // pieces_per_row = num_kv_heads * head_dim / 8.
-template <bool KF32, bool VF32>
+template <bool KF32, bool VF32, bool CF16>
 __global__ __launch_bounds__(256) void store_kvcache_kernel(
     const void* __restrict__ key, const void* __restrict__ value,
     uint4* __restrict__ k_cache, uint4* __restrict__ v_cache,
@@ -53,8 +64,8 @@ __global__ __launch_bounds__(256) void store_kvcache_kernel(
   const int piece = (int)(gid - (int64_t)token * pieces_per_row);
   const int64_t slot = slot_mapping[token];
   if (slot < 0 || slot >= num_slots) return;
-  const uint4 kb = load_piece_as_bf16<KF32>(key, gid);
-  const uint4 vb = load_piece_as_bf16<VF32>(value, gid);
+  const uint4 kb = load_piece_as_cache_type<KF32, CF16>(key, gid);
+  const uint4 vb = load_piece_as_cache_type<VF32, CF16>(value, gid);
   const int64_t dst = slot * pieces_per_row + piece;
   k_cache[dst] = kb;
   v_cache[dst] = vb;
@@ -67,11 +78,13 @@ extern "C" int nvj_store_kvcache_launch(void* stream, const void* key, const voi
                                         const int32_t* slot_mapping, int32_t num_tokens,
                                         int32_t num_kv_heads, int32_t head_dim,
                                         int64_t num_slots, int32_t k_dtype,
-                                        int32_t v_dtype) {
+                                        int32_t v_dtype, int32_t cache_dtype) {
   if (num_tokens < 0 || num_kv_heads <= 0 || head_dim <= 0 || num_slots < 0)
     return NVJ_ERR_BAD_SHAPE;
-  if ((k_dtype != NVJ_DTYPE_BF16 && k_dtype != NVJ_DTYPE_F32) ||
-      (v_dtype != NVJ_DTYPE_BF16 && v_dtype != NVJ_DTYPE_F32))
+  if (cache_dtype != NVJ_DTYPE_BF16 && cache_dtype != NVJ_DTYPE_F16) return NVJ_ERR_BAD_DTYPE;
+  // a source is float32 (rounded here) or already has the cache's type
+  if ((k_dtype != cache_dtype && k_dtype != NVJ_DTYPE_F32) ||
+      (v_dtype != cache_dtype && v_dtype != NVJ_DTYPE_F32))
     return NVJ_ERR_BAD_DTYPE;
   const int64_t row = (int64_t)num_kv_heads * head_dim;
   if (row % 8 != 0 || row / 8 > INT32_MAX) return NVJ_ERR_UNSUPPORTED;
@@ -89,17 +102,20 @@ extern "C" int nvj_store_kvcache_launch(void* stream, const void* key, const voi
   uint4* kc = static_cast<uint4*>(k_cache);
   uint4* vc = static_cast<uint4*>(v_cache);
   const bool kf = k_dtype == NVJ_DTYPE_F32, vf = v_dtype == NVJ_DTYPE_F32;
-  if (kf && vf)
-    store_kvcache_kernel<true, true><<<grid, block, 0, s>>>(key, value, kc, vc, slot_mapping,
-                                                            num_tokens, pieces, num_slots);
-  else if (kf)
-    store_kvcache_kernel<true, false><<<grid, block, 0, s>>>(key, value, kc, vc, slot_mapping,
-                                                             num_tokens, pieces, num_slots);
-  else if (vf)
-    store_kvcache_kernel<false, true><<<grid, block, 0, s>>>(key, value, kc, vc, slot_mapping,
-                                                             num_tokens, pieces, num_slots);
-  else
-    store_kvcache_kernel<false, false><<<grid, block, 0, s>>>(key, value, kc, vc, slot_mapping,
-                                                              num_tokens, pieces, num_slots);
+  const bool cf16 = cache_dtype == NVJ_DTYPE_F16;
+#define NVJ_LAUNCH_STORE(KF, VF, CF)                                                          \
+  store_kvcache_kernel<KF, VF, CF><<<grid, block, 0, s>>>(key, value, kc, vc, slot_mapping,   \
+                                                          num_tokens, pieces, num_slots)
+  switch ((kf ? 4 : 0) | (vf ? 2 : 0) | (cf16 ? 1 : 0)) {
+    case 0: NVJ_LAUNCH_STORE(false, false, false); break;   // copies: the type does not matter
+    case 1: NVJ_LAUNCH_STORE(false, false, false); break;
+    case 2: NVJ_LAUNCH_STORE(false, true, false); break;
+    case 3: NVJ_LAUNCH_STORE(false, true, true); break;
+    case 4: NVJ_LAUNCH_STORE(true, false, false); break;
+    case 5: NVJ_LAUNCH_STORE(true, false, true); break;
+    case 6: NVJ_LAUNCH_STORE(true, true, false); break;
+    default: NVJ_LAUNCH_STORE(true, true, true); break;
+  }
+#undef NVJ_LAUNCH_STORE
   return hipGetLastError() == hipSuccess ? NVJ_OK : NVJ_ERR_LAUNCH;
 }

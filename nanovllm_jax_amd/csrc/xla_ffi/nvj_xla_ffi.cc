@@ -26,6 +26,8 @@ ffi::Error to_error(int rc) {
   return ffi::Error(code, nvj_error_string(rc));
 }
 
+// The handlers are typed for the bf16 caches of the Qwen3 models the reference runs; a float16
+// cache binds the same way with F16 buffers and NVJ_DTYPE_F16.
 int dtype_code(ffi::DataType t) { return t == ffi::DataType::F32 ? NVJ_DTYPE_F32 : NVJ_DTYPE_BF16; }
 
 // operands: key, value [T, Hkv, D] (bf16 or f32), k_cache, v_cache [slots, Hkv, D] or
@@ -48,7 +50,8 @@ ffi::Error StoreKvcacheImpl(hipStream_t stream, ffi::AnyBuffer key, ffi::AnyBuff
   return to_error(nvj_store_kvcache_launch(
       stream, key.untyped_data(), value.untyped_data(), k_cache->untyped_data(),
       v_cache->untyped_data(), slot_mapping.typed_data(), (int32_t)kd[0], (int32_t)kd[1],
-      (int32_t)kd[2], num_slots, dtype_code(key.element_type()), dtype_code(value.element_type())));
+      (int32_t)kd[2], num_slots, dtype_code(key.element_type()), dtype_code(value.element_type()),
+      NVJ_DTYPE_BF16));
 }
 
 // operands: q [B, Hq, D], k_cache, v_cache [NB, bs, Hkv, D] bf16, block_tables [B, MB],
@@ -73,7 +76,7 @@ ffi::Error PagedDecodeImpl(hipStream_t stream, ffi::Buffer<ffi::DataType::BF16> 
       block_tables.typed_data(), context_lens.typed_data(), out->typed_data(),
       workspace->typed_data(), workspace->size_bytes(), (int32_t)qd[0], (int32_t)qd[1],
       (int32_t)cd[2], (int32_t)qd[2], (int32_t)cd[1], (int32_t)td[1], (int32_t)cd[0], scale,
-      chunk));
+      chunk, NVJ_DTYPE_BF16));
 }
 
 }  // namespace

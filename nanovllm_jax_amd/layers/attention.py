@@ -23,7 +23,9 @@ from .prefill_attention import variable_length_attention_prefill
 
 __all__ = ["store_kv_to_cache", "Attention"]
 
-_DTYPE_CODE = {torch.bfloat16: _lib.NVJ_DTYPE_BF16, torch.float32: _lib.NVJ_DTYPE_F32}
+_DTYPE_CODE = {torch.bfloat16: _lib.NVJ_DTYPE_BF16, torch.float32: _lib.NVJ_DTYPE_F32,
+               torch.float16: _lib.NVJ_DTYPE_F16}
+_CACHE_DTYPES = (torch.bfloat16, torch.float16)
 
 
 def _require(cond: bool, msg: str) -> None:
@@ -34,10 +36,10 @@ def _require(cond: bool, msg: str) -> None:
 def store_kv_to_cache(key, value, k_cache, v_cache, slot_mapping):
     """Scatter new K/V rows into the paged cache through ``slot_mapping``.
 
-    key, value   [num_tokens, num_kv_heads, head_dim], bf16 or float32 (float32
-                 rows are rounded to nearest-even bf16, as ``astype`` does)
+    key, value   [num_tokens, num_kv_heads, head_dim], the cache dtype or float32
+                 (float32 rows are rounded to nearest even, as ``astype`` does)
     k_cache, v_cache
-                 [num_slots, num_kv_heads, head_dim] bf16, or the 4-D
+                 [num_slots, num_kv_heads, head_dim] bf16 or float16, or the 4-D
                  [num_blocks, block_size, num_kv_heads, head_dim] view of the
                  same memory
     slot_mapping [num_tokens] int32; ``slot < 0`` skips the token, ``slot >=
@@ -57,8 +59,11 @@ def store_kv_to_cache(key, value, k_cache, v_cache, slot_mapping):
              "key and value must both be [num_tokens, num_kv_heads, head_dim]")
     _require(key.dtype in _DTYPE_CODE, f"key dtype {key.dtype} not supported")
     _require(value.dtype in _DTYPE_CODE, f"value dtype {value.dtype} not supported")
-    _require(k_cache.dtype == torch.bfloat16 and v_cache.dtype == torch.bfloat16,
-             "caches must be bf16")
+    _require(k_cache.dtype in _CACHE_DTYPES and v_cache.dtype == k_cache.dtype,
+             "caches must both be bf16 or both be float16")
+    for name, t in (("key", key), ("value", value)):
+        _require(t.dtype in (k_cache.dtype, torch.float32),
+                 f"{name} must be {k_cache.dtype} (the cache dtype) or float32, got {t.dtype}")
     _require(k_cache.shape == v_cache.shape and k_cache.dim() in (3, 4),
              "caches must have equal 3-D or 4-D shapes")
     num_tokens, num_kv_heads, head_dim = key.shape
@@ -72,7 +77,7 @@ def store_kv_to_cache(key, value, k_cache, v_cache, slot_mapping):
         code = lib.nvj_store_kvcache_launch(
             stream, key.data_ptr(), value.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(),
             slot_mapping.data_ptr(), num_tokens, num_kv_heads, head_dim, num_slots,
-            _DTYPE_CODE[key.dtype], _DTYPE_CODE[value.dtype])
+            _DTYPE_CODE[key.dtype], _DTYPE_CODE[value.dtype], _DTYPE_CODE[k_cache.dtype])
     _lib.check(code, "nvj_store_kvcache_launch")
     return k_cache, v_cache
 

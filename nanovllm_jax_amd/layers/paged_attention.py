@@ -24,11 +24,18 @@ def _require(cond: bool, msg: str) -> None:
         raise ValueError(msg)
 
 
-def _check_device_tensor(t: torch.Tensor, name: str, dtype: torch.dtype, ndim: int) -> None:
+_CACHE_DTYPE_CODE = {torch.bfloat16: _lib.NVJ_DTYPE_BF16, torch.float16: _lib.NVJ_DTYPE_F16}
+
+
+def _check_device_tensor(t: torch.Tensor, name: str, dtype, ndim: int) -> None:
+    """``dtype`` None: bf16 or float16 (the cache dtypes)."""
     _require(isinstance(t, torch.Tensor), f"{name} must be a torch.Tensor")
     _require(t.is_cuda, f"{name} must live on the GPU (got {t.device}); "
                         "the paged-decode path has no CPU implementation")
-    _require(t.dtype == dtype, f"{name} must be {dtype}, got {t.dtype}")
+    if dtype is None:
+        _require(t.dtype in _CACHE_DTYPE_CODE, f"{name} must be bfloat16 or float16, got {t.dtype}")
+    else:
+        _require(t.dtype == dtype, f"{name} must be {dtype}, got {t.dtype}")
     _require(t.dim() == ndim, f"{name} must have {ndim} dims, got shape {tuple(t.shape)}")
     _require(t.is_contiguous(), f"{name} must be contiguous")
 
@@ -72,15 +79,15 @@ def paged_attention(q, k_cache, v_cache, block_tables, context_lens, scale, bloc
                     phases: int = _lib.NVJ_PHASE_SPLITK | _lib.NVJ_PHASE_COMBINE) -> torch.Tensor:
     """Decode attention over a block-paged KV cache.
 
-    q            [batch, num_heads, head_dim]                          bf16
-    k_cache      [num_blocks, block_size, num_kv_heads, head_dim]      bf16
+    q            [batch, num_heads, head_dim]                          bf16 or float16
+    k_cache      [num_blocks, block_size, num_kv_heads, head_dim]      same dtype
     v_cache      same shape
     block_tables [batch, max_blocks] int32 (padding entries are never read)
     context_lens [batch] int32
     scale        softmax scale (Python float)
     block_size   positions per page; must equal ``k_cache.shape[1]``
 
-    Returns [batch, num_heads, head_dim] bf16.  ``chunk`` (0 = balanced split
+    Returns [batch, num_heads, head_dim] in q's dtype.  ``chunk`` (0 = balanced split
     derived from ``context_lens`` on the device; > 0 = that many positions per
     workgroup, multiple of 32; ``WHOLE_SEQUENCE`` = each sequence finished inside
     one workgroup, no workspace and no combine launch, for batches of similar
@@ -90,9 +97,9 @@ def paged_attention(q, k_cache, v_cache, block_tables, context_lens, scale, bloc
     the split-K launch, the combine launch or both (timing aid).
     """
     lib = _lib.load()
-    _check_device_tensor(q, "q", torch.bfloat16, 3)
-    _check_device_tensor(k_cache, "k_cache", torch.bfloat16, 4)
-    _check_device_tensor(v_cache, "v_cache", torch.bfloat16, 4)
+    _check_device_tensor(q, "q", None, 3)
+    _check_device_tensor(k_cache, "k_cache", q.dtype, 4)
+    _check_device_tensor(v_cache, "v_cache", q.dtype, 4)
     _check_device_tensor(block_tables, "block_tables", torch.int32, 2)
     _check_device_tensor(context_lens, "context_lens", torch.int32, 1)
     batch, num_heads, head_dim = q.shape
@@ -112,7 +119,7 @@ def paged_attention(q, k_cache, v_cache, block_tables, context_lens, scale, bloc
     if out is None:
         out = torch.empty_like(q)
     else:
-        _check_device_tensor(out, "out", torch.bfloat16, 3)
+        _check_device_tensor(out, "out", q.dtype, 3)
         _require(out.shape == q.shape and out.device == dev, "out must match q")
     need = int(lib.nvj_paged_decode_workspace_bytes(batch, num_heads, head_dim, max_blocks,
                                                     bs, num_kv_heads, chunk)) if batch and max_blocks else 0
@@ -131,6 +138,7 @@ def paged_attention(q, k_cache, v_cache, block_tables, context_lens, scale, bloc
             stream, q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(),
             block_tables.data_ptr(), context_lens.data_ptr(), out.data_ptr(),
             workspace.data_ptr(), ws_bytes, batch, num_heads, num_kv_heads, head_dim, bs,
-            max_blocks, num_blocks, float(scale), int(chunk), int(phases))
+            max_blocks, num_blocks, float(scale), int(chunk), _CACHE_DTYPE_CODE[q.dtype],
+            int(phases))
     _lib.check(code, "nvj_paged_decode_launch_phases")
     return out

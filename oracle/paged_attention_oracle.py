@@ -12,6 +12,8 @@ What pins each function (see tests/test_oracle_pinning.py):
 
 * ``f32_to_bf16_bits``          - IEEE round-to-nearest-even; cross-checked
                                   against ``torch.Tensor.to(torch.bfloat16)``.
+* ``f32_to_f16_bits``           - NumPy's IEEE conversion; cross-checked against
+                                  ``torch.Tensor.to(torch.float16)``.
 * ``store_kv_to_cache_ref``     - brute-force per-token Python loop; untouched
                                   rows unchanged; idempotence; K/V independence.
 * ``paged_decode_attention_vectorized_ref`` and ``..._per_seq``
@@ -69,6 +71,8 @@ import numpy as np
 __all__ = [
     "f32_to_bf16_bits",
     "bf16_bits_to_f32",
+    "f32_to_f16_bits",
+    "f16_bits_to_f32",
     "store_kv_to_cache_ref",
     "gather_kv_from_cache_ref",
     "paged_decode_attention_vectorized_ref",
@@ -111,6 +115,28 @@ def bf16_bits_to_f32(b: np.ndarray) -> np.ndarray:
     return (b.astype(np.uint32) << np.uint32(16)).view(np.float32)
 
 
+def f32_to_f16_bits(x: np.ndarray) -> np.ndarray:
+    """fp32 -> IEEE half, round to nearest even, as uint16 bit patterns
+    (NumPy's ``astype(float16)``; what ``astype(cache.dtype)`` of
+    ``layers/attention.py:70-71`` does for a float16 cache)."""
+    with np.errstate(over="ignore"):
+        return np.asarray(x, dtype=np.float32).astype(np.float16).view(np.uint16)
+
+
+def f16_bits_to_f32(b: np.ndarray) -> np.ndarray:
+    """IEEE half bit pattern -> fp32 (exact)."""
+    return np.ascontiguousarray(b, dtype=np.uint16).view(np.float16).astype(np.float32)
+
+
+def _codec(dtype: str):
+    """(bits -> fp32, fp32 -> bits) of a 16-bit cache dtype, "bf16" or "f16"."""
+    if dtype == "bf16":
+        return bf16_bits_to_f32, f32_to_bf16_bits
+    if dtype == "f16":
+        return f16_bits_to_f32, f32_to_f16_bits
+    raise ValueError(dtype)
+
+
 def _as_bf16_bits(x: np.ndarray) -> np.ndarray:
     """Accept fp32 values or uint16 bf16 bits; return bf16 bits."""
     if x.dtype == np.uint16:
@@ -125,11 +151,12 @@ def _as_bf16_bits(x: np.ndarray) -> np.ndarray:
 # ---------------------------------------------------------------------------
 
 def store_kv_to_cache_ref(key, value, k_cache, v_cache, slot_mapping,
-                          negative_slots: str = "reference"):
+                          negative_slots: str = "reference", dtype: str = "bf16"):
     """Restates ``store_kv_to_cache`` (``layers/attention.py:42-77``).
 
-    key, value : [T, Hkv, D] float32 values or uint16 bf16 bits
-    k_cache, v_cache : [num_slots, Hkv, D] uint16 bf16 bits (flattened cache,
+    key, value : [T, Hkv, D] float32 values or uint16 bits of the cache dtype
+    k_cache, v_cache : [num_slots, Hkv, D] uint16 bits of the cache dtype
+                 (``dtype``: "bf16" or "f16"; flattened cache,
                  ``layers/attention.py:458-463``)
     slot_mapping : [T] int32
 
@@ -148,8 +175,12 @@ def store_kv_to_cache_ref(key, value, k_cache, v_cache, slot_mapping,
     """
     if negative_slots not in ("reference", "skip"):
         raise ValueError(negative_slots)
-    kb = _as_bf16_bits(np.asarray(key))          # :70  key.astype(cache.dtype)
-    vb = _as_bf16_bits(np.asarray(value))        # :71
+    to_bits = _codec(dtype)[1]
+    key, value = np.asarray(key), np.asarray(value)
+    kb = key if key.dtype == np.uint16 else to_bits(key)          # :70  key.astype(cache.dtype)
+    vb = value if value.dtype == np.uint16 else to_bits(value)    # :71
+    if kb.dtype != np.uint16 or vb.dtype != np.uint16:
+        raise TypeError("key / value must be float32 values or uint16 bit patterns")
     slots = np.asarray(slot_mapping, dtype=np.int64)
     k_new = np.array(k_cache, dtype=np.uint16, copy=True)
     v_new = np.array(v_cache, dtype=np.uint16, copy=True)
@@ -228,13 +259,14 @@ def paged_decode_attention_vectorized_ref(q, k_cache, v_cache, block_tables,
 
 def paged_decode_attention_per_seq_ref(q, k_cache, v_cache, block_tables,
                                        context_lens, scale, block_size,
-                                       return_f32: bool = False):
+                                       return_f32: bool = False, dtype: str = "bf16"):
     """Same arithmetic as ``paged_decode_attention_vectorized_ref``
     (``layers/pallas_attention.py:146-238``), evaluated one sequence at a time
     over that sequence's own ceil(ctx/bs) pages so memory stays bounded at the
     32k-context configs.  Positions >= ctx carry weight exactly 0 in the
     reference (:225), so restricting to the live pages changes nothing but
     fp32 summation order.  ctx == 0 gives zeros (0 / (0 + 1e-9), :227).
+    ``dtype`` ("bf16" or "f16") is the 16-bit type of q, the caches and the result.
     """
     q = np.asarray(q)
     B, Hq, D = q.shape
@@ -244,6 +276,7 @@ def paged_decode_attention_per_seq_ref(q, k_cache, v_cache, block_tables,
     bt = np.asarray(block_tables)
     ctx = np.asarray(context_lens)
     scale = np.float32(scale)
+    to_f32, to_bits = _codec(dtype)
     out = np.zeros((B, Hq, D), dtype=np.float32)
     for b in range(B):
         n = int(ctx[b])
@@ -251,9 +284,9 @@ def paged_decode_attention_per_seq_ref(q, k_cache, v_cache, block_tables,
             continue
         nblk = -(-n // block_size)
         pages = np.clip(bt[b, :nblk], 0, NB - 1)                     # :185
-        k = bf16_bits_to_f32(k_cache[pages].reshape(nblk * bs, Hkv, D)[:n])
-        v = bf16_bits_to_f32(v_cache[pages].reshape(nblk * bs, Hkv, D)[:n])
-        qb = bf16_bits_to_f32(q[b]).reshape(Hkv, G, D)               # head h -> kv h // G (:197)
+        k = to_f32(k_cache[pages].reshape(nblk * bs, Hkv, D)[:n])
+        v = to_f32(v_cache[pages].reshape(nblk * bs, Hkv, D)[:n])
+        qb = to_f32(q[b]).reshape(Hkv, G, D)               # head h -> kv h // G (:197)
         s = np.einsum("kgd,skd->kgs", qb, k, dtype=np.float32) * scale
         smax = s.max(axis=-1, keepdims=True)
         e = np.exp(s - smax, dtype=np.float32)
@@ -261,7 +294,7 @@ def paged_decode_attention_per_seq_ref(q, k_cache, v_cache, block_tables,
         out[b] = np.einsum("kgs,skd->kgd", w, v, dtype=np.float32).reshape(Hq, D)
     if return_f32:
         return out
-    return f32_to_bf16_bits(out)
+    return to_bits(out)
 
 
 def paged_attention_fallback_ref(q, k_cache, v_cache, block_tables,

@@ -43,7 +43,7 @@ def test_argument_validation_without_a_gpu():
         a = dict(ok); a.update(kw)
         p = kw.get("ptr", 0x1000)
         return L(None, p, p, p, p, p, p, p, 1 << 30, a["batch"], a["Hq"], a["Hkv"], a["D"],
-                 a["bs"], a["MB"], a["NB"], 0.1, kw.get("chunk", 0))
+                 a["bs"], a["MB"], a["NB"], 0.1, kw.get("chunk", 0), kw.get("dtype", 0))
 
     assert call(D=96) == -3                # head_dim not built (128 and 64 are)
     assert call(Hq=30) == -2               # Hq % Hkv
@@ -51,17 +51,21 @@ def test_argument_validation_without_a_gpu():
     assert call(chunk=100) == -3
     assert call(chunk=-2) == -2                   # only -1 (whole sequence) is a mode below 0
     assert call(batch=-1) == -2
+    assert call(dtype=1) == -6                    # the cache is bf16 (0) or float16 (2), not f32
+    assert call(dtype=3) == -6
     assert call(batch=0) == 0              # empty batch: nothing to do
     assert call(ptr=0) == -1
     assert call(ptr=0x1004) == -4          # misaligned
     assert L(None, 0x1000, 0x1000, 0x1000, 0x1000, 0x1000, 0x1000, 0x1000, 16, 2, 32, 8, 128, 256,
-             4, 16, 0.1, 0) == -4          # workspace too small
+             4, 16, 0.1, 0, 0) == -4       # workspace too small
     S = lib.nvj_store_kvcache_launch
-    assert S(None, 0, 0, 0, 0, 0, 0, 8, 128, 1024, 0, 0) == 0       # no tokens
-    assert S(None, 0x1000, 0x1000, 0x1000, 0x1000, 0x1000, 4, 8, 128, 1024, 7, 0) == -6
-    assert S(None, 0, 0x1000, 0x1000, 0x1000, 0x1000, 4, 8, 128, 1024, 0, 0) == -1
-    assert S(None, 0x1000, 0x1000, 0x1000, 0x1000, 0x1000, 4, 3, 3, 1024, 0, 0) == -3
-    assert S(None, 0x1000, 0x1000, 0x1000, 0x1000, 0x1000, -4, 8, 128, 1024, 0, 0) == -2
+    assert S(None, 0, 0, 0, 0, 0, 0, 8, 128, 1024, 0, 0, 0) == 0       # no tokens
+    assert S(None, 0x1000, 0x1000, 0x1000, 0x1000, 0x1000, 4, 8, 128, 1024, 7, 0, 0) == -6
+    assert S(None, 0x1000, 0x1000, 0x1000, 0x1000, 0x1000, 4, 8, 128, 1024, 2, 0, 0) == -6  # f16 rows, bf16 cache
+    assert S(None, 0x1000, 0x1000, 0x1000, 0x1000, 0x1000, 4, 8, 128, 1024, 0, 0, 1) == -6  # f32 cache
+    assert S(None, 0, 0x1000, 0x1000, 0x1000, 0x1000, 4, 8, 128, 1024, 0, 0, 0) == -1
+    assert S(None, 0x1000, 0x1000, 0x1000, 0x1000, 0x1000, 4, 3, 3, 1024, 0, 0, 0) == -3
+    assert S(None, 0x1000, 0x1000, 0x1000, 0x1000, 0x1000, -4, 8, 128, 1024, 0, 0, 0) == -2
 
 
 def test_workspace_and_chunk_queries():

@@ -1,0 +1,98 @@
+"""float16 caches (the reference's cache dtype is its model dtype, and its own
+timing scripts use float16: profile_attention.py:27-30): KV store bit-exact,
+decode attention within atol/rtol 1e-2 of the oracle, in every split mode."""
+import numpy as np
+import pytest
+
+from helpers import make_problem
+
+pytestmark = pytest.mark.gpu
+
+
+def _to_f16(bits, dev):
+    import torch
+    return torch.from_numpy(np.ascontiguousarray(bits).view(np.int16)).view(torch.float16).to(dev)
+
+
+def _bits(t):
+    import torch
+    assert t.dtype == torch.float16
+    return t.detach().cpu().contiguous().view(torch.int16).numpy().view(np.uint16).copy()
+
+
+def _as_f16_problem(seed, B, Hq, Hkv, D, bs, NB, ctx, gain=1.0):
+    """The bf16 generator's values re-rounded to float16 bit patterns."""
+    from oracle.paged_attention_oracle import bf16_bits_to_f32, f32_to_f16_bits
+    q, kc, vc, bt, ctx = make_problem(seed, B, Hq, Hkv, D, bs, NB, ctx, q_gain=gain)
+    cv = lambda b: f32_to_f16_bits(bf16_bits_to_f32(b) * np.float32(1.001))   # not bf16-exact values
+    return cv(q), cv(kc), cv(vc), bt, ctx
+
+
+@pytest.mark.parametrize("chunk", [0, 64, -1])
+@pytest.mark.parametrize("Hq,Hkv,D", [(32, 8, 128), (16, 8, 128), (8, 2, 64), (32, 1, 128)])
+def test_decode_float16(Hq, Hkv, D, chunk):
+    print(f"case f16 decode Hq={Hq} Hkv={Hkv} D={D} chunk={chunk}", flush=True)
+    import torch
+    from nanovllm_jax_amd import paged_attention
+    from oracle.paged_attention_oracle import f16_bits_to_f32, paged_decode_attention_per_seq_ref
+    B, bs, NB = 9, 64, 60
+    ctx = [0, 1, 33, 64, 100, 257, 300, 31, 129]
+    q, kc, vc, bt, ctx = _as_f16_problem(800 + Hq + D, B, Hq, Hkv, D, bs, NB, ctx, gain=2.0)
+    dev = "cuda:0"
+    scale = 1.0 / np.sqrt(D)
+    out = paged_attention(_to_f16(q, dev), _to_f16(kc, dev), _to_f16(vc, dev),
+                          torch.from_numpy(bt).to(dev), torch.from_numpy(ctx).to(dev), scale, bs,
+                          chunk=chunk)
+    torch.cuda.synchronize()
+    assert out.dtype == torch.float16
+    got = f16_bits_to_f32(_bits(out)).astype(np.float64)
+    want = f16_bits_to_f32(paged_decode_attention_per_seq_ref(q, kc, vc, bt, ctx, scale, bs,
+                                                              dtype="f16")).astype(np.float64)
+    err = np.abs(got - want)
+    assert np.all(err <= 1e-2 + 1e-2 * np.abs(want)), f"max err {err.max():.3e}"
+    assert not got[0].any()                                     # ctx = 0 -> zeros
+    v_first = f16_bits_to_f32(vc[bt[1, 0], 0])                  # ctx = 1 -> the V row itself
+    assert np.array_equal(got[1], np.repeat(v_first, Hq // Hkv, axis=0))
+
+
+@pytest.mark.parametrize("k_f32,v_f32", [(True, False), (False, False), (True, True)])
+def test_store_float16_bit_exact(k_f32, v_f32):
+    print(f"case f16 store k_f32={k_f32} v_f32={v_f32}", flush=True)
+    import torch
+    from nanovllm_jax_amd import store_kv_to_cache
+    from oracle.paged_attention_oracle import f32_to_f16_bits, store_kv_to_cache_ref
+    rng = np.random.Generator(np.random.PCG64(820))
+    T, Hkv, D, slots_n = 37, 8, 128, 500
+    vals = (rng.standard_normal((2, T, Hkv, D)) * np.exp(rng.uniform(-18, 11, (2, T, Hkv, D)))
+            ).astype(np.float32)
+    vals[0, 0, 0, :6] = [65504.0, 65520.0, 1e-8, 6.0e-8, -0.0, 1 + 2.0 ** -11]   # edge values
+    kc = rng.integers(0, 0x7C00, (slots_n, Hkv, D)).astype(np.uint16)
+    vc = rng.integers(0, 0x7C00, (slots_n, Hkv, D)).astype(np.uint16)
+    slots = rng.permutation(slots_n)[:T].astype(np.int32)
+    slots[3], slots[5] = -1, slots_n + 7                          # skipped / dropped
+    dev = "cuda:0"
+    k_in = vals[0] if k_f32 else f32_to_f16_bits(vals[0])
+    v_in = vals[1] if v_f32 else f32_to_f16_bits(vals[1])
+    up = lambda a: torch.from_numpy(a).to(dev) if a.dtype == np.float32 else _to_f16(a, dev)
+    kct, vct = _to_f16(kc, dev), _to_f16(vc, dev)
+    store_kv_to_cache(up(k_in), up(v_in), kct, vct, torch.from_numpy(slots).to(dev))
+    torch.cuda.synchronize()
+    wk, wv = store_kv_to_cache_ref(k_in, v_in, kc, vc, slots, negative_slots="skip", dtype="f16")
+    assert np.array_equal(_bits(kct), wk), "K cache not bit-exact"
+    assert np.array_equal(_bits(vct), wv), "V cache not bit-exact"
+
+
+def test_mixed_dtypes_are_refused():
+    import torch
+    from nanovllm_jax_amd import paged_attention, store_kv_to_cache
+    dev = "cuda:0"
+    q = torch.zeros((1, 8, 128), dtype=torch.float16, device=dev)
+    kc = torch.zeros((2, 64, 8, 128), dtype=torch.bfloat16, device=dev)
+    bt = torch.zeros((1, 1), dtype=torch.int32, device=dev)
+    ctx = torch.ones(1, dtype=torch.int32, device=dev)
+    with pytest.raises(ValueError):
+        paged_attention(q, kc, kc, bt, ctx, 0.1, 64)               # f16 q, bf16 cache
+    k = torch.zeros((1, 8, 128), dtype=torch.float16, device=dev)
+    with pytest.raises(ValueError):
+        store_kv_to_cache(k, k, kc.view(-1, 8, 128), kc.view(-1, 8, 128),
+                          torch.zeros(1, dtype=torch.int32, device=dev))   # f16 rows, bf16 cache

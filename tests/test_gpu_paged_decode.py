@@ -282,7 +282,7 @@ def test_whole_sequence_mode_needs_no_workspace_and_ignores_garbage():
     code = lib.nvj_paged_decode_launch(
         torch.cuda.current_stream().cuda_stream, qt.data_ptr(), kt.data_ptr(), vt.data_ptr(),
         btt.data_ptr(), ct.data_ptr(), out.data_ptr(), None, 0, B, Hq, Hkv, D, bs, bt.shape[1],
-        NB, 0.09, WHOLE_SEQUENCE)
+        NB, 0.09, WHOLE_SEQUENCE, _lib.NVJ_DTYPE_BF16)
     assert code == 0
     torch.cuda.synchronize()
     assert_close_bf16(torch_to_bits(out), want, what="whole-sequence, NULL workspace, poison")

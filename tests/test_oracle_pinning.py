@@ -440,3 +440,21 @@ def test_silu_and_mul_against_float64_torch_and_closed_forms():
     assert out[0, 1] == np.float32(80.0 * -2.5)
     assert out[0, 2] == 0.0
     assert abs(out[0, 3] - 7.0 / (1 + np.exp(-1.0))) <= 2.0 ** -8 * 7
+
+
+def test_f16_rounding_against_torch_and_special_values():
+    from oracle.paged_attention_oracle import f16_bits_to_f32, f32_to_f16_bits
+    rng = np.random.Generator(np.random.PCG64(63))
+    x = np.concatenate([
+        (rng.standard_normal(200_000) * np.exp(rng.uniform(-20, 12, 200_000))).astype(np.float32),
+        np.array([0.0, -0.0, 65504.0, 65520.0, 65519.9, 1e-8, 6.0e-8, 5.96e-8, 2.98e-8, 6.1e-5,
+                  np.inf, -np.inf, 1 + 2.0 ** -11, 1 + 3 * 2.0 ** -11], np.float32)])
+    want = torch.from_numpy(x).to(torch.float16).view(torch.int16).numpy().view(np.uint16)
+    got = f32_to_f16_bits(x)
+    assert np.array_equal(got, want)
+    # ties go to even; overflow to inf; the round trip of every finite half value is exact
+    assert f32_to_f16_bits(np.array([1 + 2.0 ** -11], np.float32))[0] == 0x3C00
+    assert f32_to_f16_bits(np.array([1 + 3 * 2.0 ** -11], np.float32))[0] == 0x3C02
+    assert f32_to_f16_bits(np.array([65520.0], np.float32))[0] == 0x7C00
+    all_bits = np.arange(0x7C00, dtype=np.uint16)
+    assert np.array_equal(f32_to_f16_bits(f16_bits_to_f32(all_bits)), all_bits)
