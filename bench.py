@@ -216,6 +216,10 @@ def main():
     ap.add_argument("--dtype", default="bf16", choices=["bf16", "f16"],
                     help="cache / q / out dtype; f16 is what the reference's own timing "
                          "scripts use (no CPU baseline leg: the C restatement reads bf16)")
+    ap.add_argument("--products", default="mfma", choices=["mfma", "valu"],
+                    help="valu: time the measurement variant of the split-K kernel that does "
+                         "Q.K and P.V with vector-ALU dot products (group 4 or 8, bf16, "
+                         "balanced or whole-sequence split)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run a plain 1 GiB device-to-device copy a few times, so a "
@@ -268,9 +272,11 @@ def main():
     kflat = kc.view(-1, w.num_kv_heads, w.head_dim)
     vflat = vc.view(-1, w.num_kv_heads, w.head_dim)
 
+    variant = _lib.NVJ_PHASE_VALU_PRODUCTS if args.products == "valu" else 0
+
     def decode(phases=3):
         paged_attention(q, kc, vc, bt, ctx, w.scale, w.block_size, chunk=chunk, out=out,
-                        workspace=ws, phases=phases)
+                        workspace=ws, phases=phases | variant)
 
     def store():
         store_kv_to_cache(k_new, v_new, kflat, vflat, slots)
@@ -307,12 +313,14 @@ def main():
                                f"D={w.head_dim} page={w.block_size} "
                                f"ctx={int(w.context_lens.min())}..{int(w.context_lens.max())} "
                                f"pool={w.num_blocks} pages",
-                   "split": split_name,
+                   "split": split_name, "products": args.products,
                    "algorithmic_bytes_per_call": byts,
                    "step": "one launch" if chunk == -1 else "split-K launch + combine launch"},
         "roofline": {"bound": "hbm", "achieved": round(gbps_kernel, 1), "peak": HBM_PEAK_GBPS,
                      "unit": "GB/s", "frac": round(gbps_kernel / HBM_PEAK_GBPS, 4),
-                     "traffic": MEASURED_TRAFFIC_BYTES.get((w.name, chunk)), "kernel": kernel_name,
+                     "traffic": (MEASURED_TRAFFIC_BYTES.get((w.name, chunk))
+                                 if args.products == "mfma" else None),
+                     "kernel": kernel_name,
                      "kernel_us": round(ms_splitk * 1e3, 2)},
         # back-to-back launches of these two short kernels are paced by the host
         # (one Python -> ctypes call each), not by the kernels themselves

@@ -178,9 +178,18 @@ NVJ_API int nvj_paged_decode_launch(void* stream,
  * same arguments left in `workspace`).  Both bits = nvj_paged_decode_launch.
  * For timing one launch in isolation and for callers that want other work
  * between the two; same reference counterpart as nvj_paged_decode_launch.
+ *
+ * NVJ_PHASE_VALU_PRODUCTS, or-ed in, runs a measurement variant of the split-K
+ * kernel that computes Q.K and P.V with vector-ALU dot products instead of the
+ * matrix cores, so that the choice between the two can be timed on any
+ * workload.  Same results to the same tolerance; never selected by default.
+ * Exists for head_dim 128, bf16, exactly 4 or 8 query heads per KV head, a
+ * multiple of 8 KV heads and chunk 0 or NVJ_CHUNK_WHOLE_SEQUENCE; anything else
+ * returns NVJ_ERR_UNSUPPORTED.
  */
 #define NVJ_PHASE_SPLITK  1u
 #define NVJ_PHASE_COMBINE 2u
+#define NVJ_PHASE_VALU_PRODUCTS 4u
 NVJ_API int nvj_paged_decode_launch_phases(void* stream,
                             const void* q, const void* k_cache, const void* v_cache,
                             const int32_t* block_tables, const int32_t* context_lens,

@@ -58,6 +58,7 @@ SYMBOLS = {
 NVJ_CHUNK_WHOLE_SEQUENCE = -1
 NVJ_PHASE_SPLITK = 1
 NVJ_PHASE_COMBINE = 2
+NVJ_PHASE_VALU_PRODUCTS = 4
 
 _lock = threading.Lock()
 _lib = None

@@ -355,6 +355,297 @@ __device__ __forceinline__ void compute_segment(const DecodeArgs& a, uint4* lds,
   l_run += __shfl_xor(l_run, 32, 64);
 }
 
+// ---------------------------------------------------------------------------
+// Measurement variant: the same segment with both products on the vector ALU
+// (v_dot2c_f32_bf16) instead of the matrix cores, so that the choice between
+// the two can be timed rather than argued.  head_dim 128, bf16, exactly G = 2,
+// 4 or 8 query heads per KV head.  Same loads, same page walk, same results
+// layout as compute_segment; only the arithmetic between them differs:
+//   * Q.K: lane (pl = lane / 16, pc = lane % 16) holds dims 8*pc .. +8 of
+//     position 4*i + pl for its 8 K loads i and the same dims of all G query
+//     rows, so 4 dot2 give a 1/16 partial of score (i, h).  The 8*G partials
+//     per lane are summed over the 16 lanes of a row by a halving exchange
+//     (DPP mirror, half mirror, two quad permutes): each step a lane keeps
+//     one half of its values and adds the partner's copy of that half, which
+//     leaves lane pc with the 8*G/16 complete scores of one head.
+//   * softmax on those few scores per lane; the probabilities (bf16) and the
+//     rescale factors travel to the P.V layout through the wave's LDS tile.
+//   * P.V: lane (kg, r) holds 8 positions x 8 dims of V, transposed in-lane
+//     into (position pair) x dim words as in the MFMA path, then 4 dot2 per
+//     (head, dim) against the matching probability pairs; the four position
+//     groups kg are summed once at the end.
+// ---------------------------------------------------------------------------
+__device__ __forceinline__ float dot2_bf16(uint32_t a, uint32_t b, float c) {
+  typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2;
+  return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2, a),
+                                         __builtin_bit_cast(bf16x2, b), c, false);
+}
+
+// value of the lane that DPP control CTRL pairs this lane with (same row of 16)
+template <int CTRL> __device__ __forceinline__ float dpp_partner(float x) {
+  return __builtin_bit_cast(
+      float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), CTRL, 0xF, 0xF, false));
+}
+
+// One halving step over v[0 .. 2*HALF): the lane whose `upper` is false keeps
+// the even entries, its partner (upper true) the odd ones; each adds the
+// partner's copy of what it keeps.  Result in v[0 .. HALF).
+template <int CTRL, int HALF, int N>
+__device__ __forceinline__ void halve_across(float (&v)[N], bool upper) {
+#pragma unroll
+  for (int j = 0; j < HALF; ++j) {
+    const float keep = upper ? v[2 * j + 1] : v[2 * j];
+    const float send = upper ? v[2 * j] : v[2 * j + 1];
+    v[j] = keep + dpp_partner<CTRL>(send);
+  }
+}
+
+constexpr int kDppQuadXor1 = 0xB1;      // quad_perm [1,0,3,2]
+constexpr int kDppQuadXor2 = 0x4E;      // quad_perm [2,3,0,1]
+constexpr int kDppRowMirror = 0x140;    // lane i <-> 15 - i
+constexpr int kDppHalfMirror = 0x141;   // lane i <-> i ^ 7
+
+template <int G>
+__device__ __forceinline__ void compute_segment_valu(const DecodeArgs& a, uint4* lds, int b,
+                                                     int kvh, int t0, int t1, int lane,
+                                                     f32x4 (&acc_out)[8], float& m_out,
+                                                     float& l_out) {
+  static_assert(G == 2 || G == 4 || G == 8, "vector-ALU variant: 2, 4 or 8 query heads");
+  constexpr int D = 128;
+  using H = HeadDim<D>;
+  // the 8 K loads of a step are scored in batches of LB loads = NB partial
+  // scores per lane, which the exchange turns into NB / 16 complete ones
+  constexpr int LB = G <= 4 ? 8 : 32 / G;   // K loads per batch
+  constexpr int NB = LB * G;                // partial scores per lane and batch (16 or 32)
+  constexpr int CB = NB / 16;               // complete scores per lane and batch
+  constexpr int NS = 8 / LB * CB;           // complete scores per lane and step
+  const int r = lane & 15, kg = lane >> 4;   // (piece, position group) in either layout
+  const char* __restrict__ k_cache = a.k_cache;
+  const char* __restrict__ v_cache = a.v_cache;
+  const int block_size = a.block_size, num_blocks = a.num_blocks;
+  const float scale_log2e = a.scale_log2e;
+  const int nsteps = (t1 - t0 + kStep - 1) / kStep;
+
+  // wave-private LDS: probabilities [G][32] bf16, rescale factors [G] f32,
+  // and at the end of the segment the results [G][128] f32 + (max, sum) [G][2]
+  uint16_t* lds_p = reinterpret_cast<uint16_t*>(lds);
+  float* lds_alpha = reinterpret_cast<float*>(lds) + 256;   // byte 1024
+  float* lds_o = reinterpret_cast<float*>(lds) + 512;       // byte 2048
+  float* lds_ml = lds_o + G * D;
+  static_assert((512 + 8 * 128 + 16) * 4 <= kStep * H::kLdsRowPieces * 16, "fits the K tile");
+
+  uint4 qv[G];   // dims 8*r .. +8 of every query row of the group
+#pragma unroll
+  for (int h = 0; h < G; ++h)
+    qv[h] = a.q[((int64_t)b * a.num_heads + (int64_t)kvh * G + h) * H::kPieces + r];
+
+  // the scores this lane owns after the exchange: entry c of a batch is partial
+  // index n = low + 16 * c, low = the bits of r in reverse order; n = h + G * i
+  // with i the load inside the batch
+  const int low = ((r >> 3) & 1) | ((r >> 1) & 2) | ((r << 1) & 4) | ((r << 3) & 8);
+  const int my_h = low % G;
+  int my_pos[NS];   // position inside the step, entry = batch * CB + c
+#pragma unroll
+  for (int bt = 0; bt < 8 / LB; ++bt)
+#pragma unroll
+    for (int c = 0; c < CB; ++c) my_pos[bt * CB + c] = 4 * (bt * LB + (low + 16 * c) / G) + kg;
+  // one lane per head publishes that head's values: the first of those that share it
+  const bool publisher = kg == 0 && (r & (16 / G - 1)) == 0;
+
+  const uint32_t row_bytes = (uint32_t)a.cache_kv_heads * (D * 2);
+  const int64_t head_bytes = (int64_t)(kvh / a.kv_rep) * (D * 2);
+  const const_i32_ptr table = as_constant(a.block_tables + (int64_t)b * a.max_blocks);
+  auto step_base = [&](int step) -> int64_t {
+    const int ts = t0 + step * kStep;
+    const int page = ts / block_size;
+    const int phys = min(max(table[page], 0), num_blocks - 1);
+    return ((int64_t)phys * block_size + (ts - page * block_size)) * row_bytes + head_bytes;
+  };
+
+  uint4 kreg[H::kKLoads], vreg[8];
+  {
+    const int64_t off = step_base(0);
+    const int last = min(kStep, t1 - t0) - 1;
+    issue_k_loads<true, D>(kreg, k_cache + off, lane, last, row_bytes);
+    issue_v_loads<true, D>(vreg, v_cache + off, kg, r, last, row_bytes);
+  }
+
+  float acc[G][8];   // O[head h][dim 8*r + jd], this lane's position group only
+#pragma unroll
+  for (int h = 0; h < G; ++h)
+#pragma unroll
+    for (int jd = 0; jd < 8; ++jd) acc[h][jd] = 0.f;
+  float m_run = kNegBig, l_run = 0.f;   // of head my_h; l_run is this lane's share
+
+  for (int step = 0; step < nsteps; ++step) {
+    const int nvalid = min(kStep, t1 - (t0 + step * kStep));
+    const bool more = step + 1 < nsteps;
+    int64_t next_off = 0;
+    int next_last = kStep - 1;
+    if (more) {
+      next_off = step_base(step + 1);
+      next_last = min(kStep, t1 - (t0 + (step + 1) * kStep)) - 1;
+    }
+
+    // ---- scores, batch by batch, then next K loads ----
+    float v[NS];
+#pragma unroll
+    for (int bt = 0; bt < 8 / LB; ++bt) {
+      float part[NB];
+#pragma unroll
+      for (int i = 0; i < LB; ++i)
+#pragma unroll
+        for (int h = 0; h < G; ++h) {
+          const uint4 kk = kreg[bt * LB + i];
+          float s = dot2_bf16(kk.x, qv[h].x, 0.f);
+          s = dot2_bf16(kk.y, qv[h].y, s);
+          s = dot2_bf16(kk.z, qv[h].z, s);
+          part[h + G * i] = dot2_bf16(kk.w, qv[h].w, s);
+        }
+      halve_across<kDppRowMirror, NB / 2>(part, (r & 8) != 0);
+      halve_across<kDppHalfMirror, NB / 4>(part, (r & 4) != 0);
+      halve_across<kDppQuadXor2, NB / 8>(part, (r & 2) != 0);
+      halve_across<kDppQuadXor1, NB / 16>(part, (r & 1) != 0);
+#pragma unroll
+      for (int c = 0; c < CB; ++c) v[bt * CB + c] = part[c];
+    }
+    if (more) {
+      if (next_last == kStep - 1)
+        issue_k_loads<false, D>(kreg, k_cache + next_off, lane, next_last, row_bytes);
+      else
+        issue_k_loads<true, D>(kreg, k_cache + next_off, lane, next_last, row_bytes);
+    }
+
+    // ---- online softmax of head my_h over the lanes that share it ----
+    float mx = kNegBig;
+#pragma unroll
+    for (int c = 0; c < NS; ++c) {
+      if (my_pos[c] >= nvalid) v[c] = kNegBig;
+      mx = fmaxf(mx, v[c]);
+    }
+    mx = fmaxf(mx, dpp_partner<kDppQuadXor1>(mx));
+    if (G <= 4) mx = fmaxf(mx, dpp_partner<kDppQuadXor2>(mx));
+    if (G <= 2) mx = fmaxf(mx, dpp_partner<kDppHalfMirror>(mx));
+    mx = wave_xor_max(mx, 16);
+    mx = wave_xor_max(mx, 32);
+    const float m_new = fmaxf(m_run, mx);
+    const float alpha = __builtin_amdgcn_exp2f((m_run - m_new) * scale_log2e);
+    const float mneg = -m_new * scale_log2e;
+    m_run = m_new;
+    float psum = 0.f;
+#pragma unroll
+    for (int c = 0; c < NS; ++c) {
+      float p = __builtin_amdgcn_exp2f(fmaf(v[c], scale_log2e, mneg));
+      if (my_pos[c] >= nvalid) p = 0.f;   // exactly 0 whatever the scale
+      psum += p;
+      lds_p[my_h * kStep + my_pos[c]] = (uint16_t)(Elem<false>::pack2(p, 0.f) & 0xFFFFu);
+    }
+    l_run = fmaf(l_run, alpha, psum);
+    const bool rescale = __builtin_amdgcn_ballot_w64(alpha != 1.0f) != 0ull;
+    if (rescale && publisher) lds_alpha[my_h] = alpha;
+    // the wave's own LDS accesses complete in order; the fence keeps the
+    // compiler from moving the reads below ahead of the writes above
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+
+    // ---- V: in-lane 8x8 transpose (positions x dims), then next V loads ----
+    uint4 vt[8];
+#pragma unroll
+    for (int w = 0; w < 4; ++w) {
+      uint32_t vw[8];
+#pragma unroll
+      for (int j = 0; j < 8; ++j)
+        vw[j] = w == 0 ? vreg[j].x : w == 1 ? vreg[j].y : w == 2 ? vreg[j].z : vreg[j].w;
+      vt[2 * w].x = __builtin_amdgcn_perm(vw[1], vw[0], 0x05040100u);
+      vt[2 * w].y = __builtin_amdgcn_perm(vw[3], vw[2], 0x05040100u);
+      vt[2 * w].z = __builtin_amdgcn_perm(vw[5], vw[4], 0x05040100u);
+      vt[2 * w].w = __builtin_amdgcn_perm(vw[7], vw[6], 0x05040100u);
+      vt[2 * w + 1].x = __builtin_amdgcn_perm(vw[1], vw[0], 0x07060302u);
+      vt[2 * w + 1].y = __builtin_amdgcn_perm(vw[3], vw[2], 0x07060302u);
+      vt[2 * w + 1].z = __builtin_amdgcn_perm(vw[5], vw[4], 0x07060302u);
+      vt[2 * w + 1].w = __builtin_amdgcn_perm(vw[7], vw[6], 0x07060302u);
+    }
+    if (more) {
+      if (next_last == kStep - 1)
+        issue_v_loads<false, D>(vreg, v_cache + next_off, kg, r, next_last, row_bytes);
+      else
+        issue_v_loads<true, D>(vreg, v_cache + next_off, kg, r, next_last, row_bytes);
+    }
+
+    // ---- O = alpha * O + P . V for every head of the group ----
+#pragma unroll
+    for (int h = 0; h < G; ++h) {
+      // probabilities of positions 4*kg .. +4 and 16 + 4*kg .. +4, as pairs
+      const uint2 plo = *reinterpret_cast<const uint2*>(lds_p + h * kStep + 4 * kg);
+      const uint2 phi = *reinterpret_cast<const uint2*>(lds_p + h * kStep + 16 + 4 * kg);
+      if (rescale) {
+        const float al = lds_alpha[h];
+#pragma unroll
+        for (int jd = 0; jd < 8; ++jd) acc[h][jd] *= al;
+      }
+#pragma unroll
+      for (int jd = 0; jd < 8; ++jd) {
+        float o = dot2_bf16(vt[jd].x, plo.x, acc[h][jd]);
+        o = dot2_bf16(vt[jd].y, plo.y, o);
+        o = dot2_bf16(vt[jd].z, phi.x, o);
+        acc[h][jd] = dot2_bf16(vt[jd].w, phi.y, o);
+      }
+    }
+    // the next step's writes must not overtake these reads
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+  }
+
+  // ---- totals: the sum of head my_h over the lanes that share it; O over the
+  // four position groups ----
+  l_run += dpp_partner<kDppQuadXor1>(l_run);
+  if (G <= 4) l_run += dpp_partner<kDppQuadXor2>(l_run);
+  if (G <= 2) l_run += dpp_partner<kDppHalfMirror>(l_run);
+  l_run += __shfl_xor(l_run, 16, 64);
+  l_run += __shfl_xor(l_run, 32, 64);
+#pragma unroll
+  for (int h = 0; h < G; ++h)
+#pragma unroll
+    for (int jd = 0; jd < 8; ++jd) {
+      float o = acc[h][jd];
+      o += __shfl_xor(o, 16, 64);
+      o += __shfl_xor(o, 32, 64);
+      acc[h][jd] = o;
+    }
+
+  // ---- hand over in the layout the MFMA path leaves: lane (r = head, kg)
+  // holds O[head r][dim 32*kg + 8*e + jd] in acc_out[jd][e] ----
+  if (kg == 0) {
+#pragma unroll
+    for (int h = 0; h < G; ++h) {
+      float4* dst = reinterpret_cast<float4*>(lds_o + h * D + 8 * r);
+      dst[0] = make_float4(acc[h][0], acc[h][1], acc[h][2], acc[h][3]);
+      dst[1] = make_float4(acc[h][4], acc[h][5], acc[h][6], acc[h][7]);
+    }
+  }
+  if (publisher) {
+    lds_ml[2 * my_h] = m_run;
+    lds_ml[2 * my_h + 1] = l_run;
+  }
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+  __builtin_amdgcn_wave_barrier();
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+  const int hr = min(r, G - 1);   // padding lanes read a real head and are ignored later
+#pragma unroll
+  for (int e = 0; e < 4; ++e) {
+    const float4* src = reinterpret_cast<const float4*>(lds_o + hr * D + 32 * kg + 8 * e);
+    const float4 x = src[0], y = src[1];
+    acc_out[0][e] = x.x; acc_out[1][e] = x.y; acc_out[2][e] = x.z; acc_out[3][e] = x.w;
+    acc_out[4][e] = y.x; acc_out[5][e] = y.y; acc_out[6][e] = y.z; acc_out[7][e] = y.w;
+  }
+  m_out = lds_ml[2 * hr];
+  l_out = lds_ml[2 * hr + 1];
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+  __builtin_amdgcn_wave_barrier();
+}
+
 // Normalised bf16 result of a whole sequence straight to `out`.
 template <int D, bool F16>
 __device__ __forceinline__ void write_output(const DecodeArgs& a, int b, int kvh, int lane,
@@ -395,13 +686,14 @@ __device__ __forceinline__ void write_partial(const DecodeArgs& a, int64_t slot,
 
 // compute_segment, then: `direct` (the segment is the whole sequence) -> out,
 // otherwise -> partial slot `slot`.
-template <int D, bool F16>
+template <int D, bool F16, int VG = 0>
 __device__ __forceinline__ void run_segment(const DecodeArgs& a, uint4* lds, int b, int kvh,
                                             int t0, int t1, int64_t slot, bool direct,
                                             int lane) {
   f32x4 acc[8];
   float m_run, l_run;
-  compute_segment<D, F16>(a, lds, b, kvh, t0, t1, lane, acc, m_run, l_run);
+  if constexpr (VG > 0) compute_segment_valu<VG>(a, lds, b, kvh, t0, t1, lane, acc, m_run, l_run);
+  else compute_segment<D, F16>(a, lds, b, kvh, t0, t1, lane, acc, m_run, l_run);
   if (direct) write_output<D, F16>(a, b, kvh, lane, acc, l_run);
   else write_partial<D>(a, slot, kvh, lane, acc, m_run, l_run);
 }
@@ -436,7 +728,9 @@ __global__ __launch_bounds__(NW * 64) void paged_decode_splitk_kernel(DecodeArgs
 // wave's K tile is free by then and exactly holds its 34 floats per lane) and
 // the wave of part 0 merges them and writes the output.  Meant for batches of
 // similar lengths: a workgroup's time follows its sequence's length.
-template <int NW, int D, bool F16>
+// VG > 0 selects the vector-ALU measurement variant for exactly VG query heads
+// per KV head (head_dim 128, bf16 only).
+template <int NW, int D, bool F16, int VG = 0>
 __global__ __launch_bounds__(NW * 64) void paged_decode_whole_kernel(DecodeArgs a, int hpw) {
   using H = HeadDim<D>;
   __shared__ uint4 k_tile[NW][kStep * H::kLdsRowPieces];
@@ -460,9 +754,14 @@ __global__ __launch_bounds__(NW * 64) void paged_decode_whole_kernel(DecodeArgs 
 #pragma unroll
   for (int jd = 0; jd < 8; ++jd) acc[jd] = f32x4{0.f, 0.f, 0.f, 0.f};
   float m_run = kNegBig, l_run = 0.f;
-  if (s1 > s0)
-    compute_segment<D, F16>(a, k_tile[wave], b, kvh, s0 * kStep, min(ctx, s1 * kStep), lane, acc,
-                            m_run, l_run);
+  if (s1 > s0) {
+    if constexpr (VG > 0)
+      compute_segment_valu<VG>(a, k_tile[wave], b, kvh, s0 * kStep, min(ctx, s1 * kStep), lane,
+                               acc, m_run, l_run);
+    else
+      compute_segment<D, F16>(a, k_tile[wave], b, kvh, s0 * kStep, min(ctx, s1 * kStep), lane,
+                              acc, m_run, l_run);
+  }
   if (parts > 1) {
     // value v of lane l at float v * kLanesWithDims + l of the wave's tile
     const bool holds_dims = lane < kLanesWithDims;
@@ -523,7 +822,7 @@ __device__ __forceinline__ int wave_inclusive_scan(int x) {
 // never needs the lengths.  Workgroup 0 also leaves the exclusive prefix sums
 // (steps before each sequence, total at [batch]) in `prefix` for the combine
 // pass.  grid.x = num_wgs, grid.y = num_kv_heads / NW, block = NW * 64.
-template <int NW, int D, bool F16>
+template <int NW, int D, bool F16, int VG = 0>
 __global__ __launch_bounds__(NW * 64) void paged_decode_balanced_kernel(DecodeArgs a, int batch,
                                                                         int num_wgs,
                                                                         int min_steps,
@@ -628,8 +927,8 @@ __global__ __launch_bounds__(NW * 64) void paged_decode_balanced_kernel(DecodeAr
     const int t0 = __builtin_amdgcn_readfirstlane((pos - before) * kStep);
     const int t1 = __builtin_amdgcn_readfirstlane(min(ctx, (seg_end - before) * kStep));
     const bool direct = pos == before && seg_end == before + nb;
-    run_segment<D, F16>(a, k_tile[wave], sb, blockIdx.y * NW + wave, t0, t1, (int64_t)(g + sb),
-                        direct, lane);
+    run_segment<D, F16, VG>(a, k_tile[wave], sb, blockIdx.y * NW + wave, t0, t1,
+                            (int64_t)(g + sb), direct, lane);
     pos = seg_end;
   }
 }
@@ -844,6 +1143,11 @@ extern "C" int nvj_paged_decode_launch_phases(void* stream, const void* q, const
        reinterpret_cast<uintptr_t>(v_cache) | reinterpret_cast<uintptr_t>(out) |
        (whole ? 0 : reinterpret_cast<uintptr_t>(workspace))) & 15u)   // unused in whole mode
     return NVJ_ERR_WORKSPACE;
+  // the vector-ALU measurement variant exists for one shape family only
+  const bool valu = (phases & NVJ_PHASE_VALU_PRODUCTS) != 0;
+  if (valu && (head_dim != 128 || f16 || kv_rep != 1 || (group != 4 && group != 8) ||
+               num_kv_heads % 8 != 0 || chunk > 0))
+    return NVJ_ERR_UNSUPPORTED;
   hipStream_t s = static_cast<hipStream_t>(stream);
 
   DecodeArgs a;
@@ -870,7 +1174,9 @@ extern "C" int nvj_paged_decode_launch_phases(void* stream, const void* q, const
     if (!(phases & NVJ_PHASE_SPLITK)) return NVJ_OK;   // there is no second pass
     const int hpw = whole_sequence_heads_per_workgroup(batch, num_kv_heads);
     const dim3 grid((unsigned)(batch * (num_kv_heads / hpw)));
-    if (head_dim == 128 && !f16) paged_decode_whole_kernel<8, 128, false><<<grid, dim3(512), 0, s>>>(a, hpw);
+    if (valu && group == 4) paged_decode_whole_kernel<8, 128, false, 4><<<grid, dim3(512), 0, s>>>(a, hpw);
+    else if (valu) paged_decode_whole_kernel<8, 128, false, 8><<<grid, dim3(512), 0, s>>>(a, hpw);
+    else if (head_dim == 128 && !f16) paged_decode_whole_kernel<8, 128, false><<<grid, dim3(512), 0, s>>>(a, hpw);
     else if (head_dim == 128) paged_decode_whole_kernel<8, 128, true><<<grid, dim3(512), 0, s>>>(a, hpw);
     else if (!f16) paged_decode_whole_kernel<8, 64, false><<<grid, dim3(512), 0, s>>>(a, hpw);
     else paged_decode_whole_kernel<8, 64, true><<<grid, dim3(512), 0, s>>>(a, hpw);
@@ -913,7 +1219,14 @@ extern "C" int nvj_paged_decode_launch_phases(void* stream, const void* q, const
 #define NVJ_LAUNCH_BALANCED(NWV, DV, F16V)                                      \
   paged_decode_balanced_kernel<NWV, DV, F16V><<<grid, dim3(NWV * 64), 0, s>>>( \
       a, batch, plan.num_wgs, kMinBalancedSteps, prefix)
-        NVJ_FOR_SHAPE(NVJ_LAUNCH_BALANCED)
+        if (valu && group == 4)
+          paged_decode_balanced_kernel<8, 128, false, 4><<<grid, dim3(512), 0, s>>>(
+              a, batch, plan.num_wgs, kMinBalancedSteps, prefix);
+        else if (valu)
+          paged_decode_balanced_kernel<8, 128, false, 8><<<grid, dim3(512), 0, s>>>(
+              a, batch, plan.num_wgs, kMinBalancedSteps, prefix);
+        else
+          NVJ_FOR_SHAPE(NVJ_LAUNCH_BALANCED)
 #undef NVJ_LAUNCH_BALANCED
       } else {
         const dim3 grid((unsigned)(batch * plan.max_chunks), gy);

@@ -58,6 +58,14 @@ def test_argument_validation_without_a_gpu():
     assert call(ptr=0x1004) == -4          # misaligned
     assert L(None, 0x1000, 0x1000, 0x1000, 0x1000, 0x1000, 0x1000, 0x1000, 16, 2, 32, 8, 128, 256,
              4, 16, 0.1, 0, 0) == -4       # workspace too small
+    # the vector-ALU measurement variant exists for group 4 or 8, head_dim 128, bf16 only
+    P = lib.nvj_paged_decode_launch_phases
+    valu = _lib.NVJ_PHASE_SPLITK | _lib.NVJ_PHASE_COMBINE | _lib.NVJ_PHASE_VALU_PRODUCTS
+    x = 0x1000
+    assert P(None, x, x, x, x, x, x, x, 1 << 30, 2, 16, 8, 128, 256, 4, 16, 0.1, 0, 0, valu) == -3
+    assert P(None, x, x, x, x, x, x, x, 1 << 30, 2, 32, 8, 128, 256, 4, 16, 0.1, 0, 2, valu) == -3
+    assert P(None, x, x, x, x, x, x, x, 1 << 30, 2, 32, 8, 128, 256, 4, 16, 0.1, 256, 0, valu) == -3
+    assert P(None, x, x, x, x, x, x, x, 1 << 30, 0, 32, 8, 128, 256, 4, 16, 0.1, 0, 0, valu) == 0
     S = lib.nvj_store_kvcache_launch
     assert S(None, 0, 0, 0, 0, 0, 0, 8, 128, 1024, 0, 0, 0) == 0       # no tokens
     assert S(None, 0x1000, 0x1000, 0x1000, 0x1000, 0x1000, 4, 8, 128, 1024, 7, 0, 0) == -6

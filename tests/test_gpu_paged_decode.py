@@ -366,3 +366,54 @@ def test_more_than_16_query_heads_per_kv_head(Hq, Hkv, D, chunk):
     got = run_hip(q, kc, vc, bt, ctx, scale, bs, chunk)
     want = oracle(q, kc, vc, bt, ctx, scale, bs)
     assert_close_bf16(got, want, what=f"large group Hq={Hq} Hkv={Hkv} chunk={chunk}")
+
+
+# ---- the vector-ALU measurement variant (phases | NVJ_PHASE_VALU_PRODUCTS) ----
+def run_hip_valu(q, kc, vc, bt, ctx, scale, bs, chunk):
+    import torch
+    from nanovllm_jax_amd import _lib, paged_attention
+    dev = "cuda:0"
+    out = paged_attention(bits_to_torch(q, dev), bits_to_torch(kc, dev), bits_to_torch(vc, dev),
+                          torch.from_numpy(bt).to(dev), torch.from_numpy(ctx).to(dev),
+                          scale, bs, chunk=chunk,
+                          phases=_lib.NVJ_PHASE_SPLITK | _lib.NVJ_PHASE_COMBINE |
+                          _lib.NVJ_PHASE_VALU_PRODUCTS)
+    torch.cuda.synchronize()
+    return torch_to_bits(out)
+
+
+@pytest.mark.parametrize("chunk", [0, -1])
+@pytest.mark.parametrize("B,Hq,Hkv", [(7, 32, 8), (7, 64, 8), (70, 64, 16), (300, 32, 8)])
+def test_vector_alu_variant_matches_the_oracle(B, Hq, Hkv, chunk):
+    print(f"case vector-ALU variant B={B} Hq={Hq} Hkv={Hkv} chunk={chunk}", flush=True)
+    rng = np.random.Generator(np.random.PCG64(950 + B + Hq))
+    bs = 64
+    ctx = rng.integers(1, 700, size=B)
+    ctx[:7] = [0, 1, 31, 33, 64, 257, 1000]
+    NB = int((-(-ctx // bs)).sum()) + 2
+    q, kc, vc, bt, ctx = make_problem(950 + B, B, Hq, Hkv, 128, bs, NB, ctx, q_gain=2.0)
+    scale = 1.0 / np.sqrt(128)
+    want = oracle(q, kc, vc, bt, ctx, scale, bs)
+    got = run_hip_valu(q, kc, vc, bt, ctx, scale, bs, chunk)
+    assert_close_bf16(got, want, what=f"vector-ALU variant chunk={chunk}")
+    assert not got[0].any(), "ctx=0 must give zeros"
+    assert np.array_equal(got[1], np.repeat(vc[bt[1, 0], 0], Hq // Hkv, axis=0))
+    assert_close_bf16(got, run_hip(q, kc, vc, bt, ctx, scale, bs, chunk), what="vs MFMA")
+
+
+def test_vector_alu_variant_refuses_other_shapes():
+    import torch
+    from nanovllm_jax_amd import _lib, paged_attention
+    dev = "cuda:0"
+    flags = _lib.NVJ_PHASE_SPLITK | _lib.NVJ_PHASE_COMBINE | _lib.NVJ_PHASE_VALU_PRODUCTS
+    bt = torch.zeros((1, 1), dtype=torch.int32, device=dev)
+    ctx = torch.ones(1, dtype=torch.int32, device=dev)
+    for Hq, Hkv, D, dt, chunk in [(16, 8, 128, torch.bfloat16, 0),     # group 2
+                                  (32, 8, 64, torch.bfloat16, 0),      # head_dim 64
+                                  (32, 8, 128, torch.float16, 0),      # float16
+                                  (16, 4, 128, torch.bfloat16, 0),     # 4 KV heads
+                                  (32, 8, 128, torch.bfloat16, 64)]:   # fixed chunks
+        q = torch.zeros((1, Hq, D), dtype=dt, device=dev)
+        kc = torch.zeros((2, 64, Hkv, D), dtype=dt, device=dev)
+        with pytest.raises(_lib.NativeLibraryError, match="unsupported"):
+            paged_attention(q, kc, kc, bt, ctx, 0.1, 64, chunk=chunk, phases=flags)
