@@ -269,18 +269,18 @@ NVJ_API int nvj_advance_decode_launch(void* stream, const void* next_tokens,
  * variable_length_attention_prefill (layers/attention.py:135-279) as called
  * from Attention._prefill_attention (layers/attention.py:331-364).
  *
- *   q   [total_q_tokens, num_heads, head_dim]     bf16
- *   k,v [total_k_tokens, num_kv_heads, head_dim]  bf16 (total_k_tokens =
+ *   q   [total_q_tokens, num_heads, head_dim]     `dtype`: NVJ_DTYPE_BF16 or NVJ_DTYPE_F16
+ *   k,v [total_k_tokens, num_kv_heads, head_dim]  `dtype` (total_k_tokens =
  *       cu_seqlens_k[batch]); the new rows of the prompts, not the paged cache
  *   cu_seqlens_q, cu_seqlens_k [batch + 1] int32, device memory
- *   out [total_q_tokens, num_heads, head_dim]     bf16
+ *   out [total_q_tokens, num_heads, head_dim]     `dtype`
  *
  * Sequence i owns q rows [cu_q[i], cu_q[i+1]) and k/v rows [cu_k[i], cu_k[i+1]).
  * Query position p (counted from the start of its sequence) attends key
  * positions <= p of the same sequence (the reference's q_pos >= k_pos mask,
  * :232-243, combined with the padding masks); query head h uses kv head
  * h / (num_heads / num_kv_heads); fp32 softmax and accumulation, probabilities
- * rounded to bf16 for the PV product, bf16 result.  A query row with no visible
+ * rounded to `dtype` for the PV product, result in `dtype`.  A query row with no visible
  * key (its sequence has no k rows) gives zeros.  The static max_seqlen_q /
  * max_seqlen_k of the reference are not needed: nothing is padded.
  * total_q_tokens bounds the launch and must be >= cu_seqlens_q[batch].
@@ -290,7 +290,7 @@ NVJ_API int nvj_prefill_attention_launch(void* stream, const void* q, const void
                             const void* v, const int32_t* cu_seqlens_q,
                             const int32_t* cu_seqlens_k, void* out,
                             int32_t total_q_tokens, int32_t batch, int32_t num_heads,
-                            int32_t num_kv_heads, int32_t head_dim, float scale);
+                            int32_t num_kv_heads, int32_t head_dim, float scale, int32_t dtype);
 
 /*
  * RMSNorm over the last dimension, optionally fused with the residual add.

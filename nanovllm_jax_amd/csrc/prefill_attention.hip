@@ -57,11 +57,35 @@ constexpr float kLog2e = 1.4426950408889634f;
 
 __device__ __forceinline__ bf16x8 as_bf16x8(uint4 v) { return __builtin_bit_cast(bf16x8, v); }
 
-__device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi) {
-  typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2;
-  bf16x2 p = {(__bf16)lo, (__bf16)hi};
-  return __builtin_bit_cast(uint32_t, p);
-}
+// The element type of q, k, v and out: bf16 (F16 = false) or IEEE half.  The
+// kernel moves 16-bit patterns (held as bf16x8 whatever they mean); only the
+// matrix instruction, the rounding of probabilities and output and the
+// constant 1 depend on the type.
+typedef __attribute__((ext_vector_type(8))) _Float16 f16x8;
+template <bool F16> struct Elem;
+template <> struct Elem<false> {
+  static constexpr uint32_t kOnes = 0x3F803F80u;   // two bf16 ones
+  static __device__ __forceinline__ f32x4 mfma(bf16x8 a, bf16x8 b, f32x4 c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0);
+  }
+  static __device__ __forceinline__ uint32_t pack2(float lo, float hi) {
+    typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2;
+    bf16x2 p = {(__bf16)lo, (__bf16)hi};
+    return __builtin_bit_cast(uint32_t, p);
+  }
+};
+template <> struct Elem<true> {
+  static constexpr uint32_t kOnes = 0x3C003C00u;   // two half ones
+  static __device__ __forceinline__ f32x4 mfma(bf16x8 a, bf16x8 b, f32x4 c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8, a),
+                                                  __builtin_bit_cast(f16x8, b), c, 0, 0, 0);
+  }
+  static __device__ __forceinline__ uint32_t pack2(float lo, float hi) {
+    typedef __attribute__((ext_vector_type(2))) _Float16 f16x2;
+    f16x2 p = {(_Float16)lo, (_Float16)hi};   // round to nearest even
+    return __builtin_bit_cast(uint32_t, p);
+  }
+};
 
 typedef const __attribute__((address_space(4))) int32_t* const_i32_ptr;
 
@@ -156,6 +180,7 @@ __device__ __forceinline__ float max_of8(const f32x4& a, const f32x4& b) {
 
 // S^T of one 32-key tile against both column groups (16 query rows each):
 // sc[g][h] holds keys 16*h + 4*kg + e of the tile for query row r of group g.
+template <bool F16>
 __device__ __forceinline__ void scores_of_tile(lds_ptr kt, const bf16x8 (&qreg)[kGroups][4],
                                                f32x4 (&sc)[kGroups][2], int r, int kg) {
   bf16x8 ka[2][4];
@@ -171,8 +196,8 @@ __device__ __forceinline__ void scores_of_tile(lds_ptr kt, const bf16x8 (&qreg)[
     sc[g][0] = sc[g][1] = f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
     for (int s = 0; s < 4; ++s) {
-      sc[g][0] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ka[0][s], qreg[g][s], sc[g][0], 0, 0, 0);
-      sc[g][1] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ka[1][s], qreg[g][s], sc[g][1], 0, 0, 0);
+      sc[g][0] = Elem<F16>::mfma(ka[0][s], qreg[g][s], sc[g][0]);
+      sc[g][1] = Elem<F16>::mfma(ka[1][s], qreg[g][s], sc[g][1]);
     }
   }
 }
@@ -188,6 +213,7 @@ __device__ __forceinline__ void scores_of_tile(lds_ptr kt, const bf16x8 (&qreg)[
 // Every element of lacc[g] of a lane is the sum over all 32 keys of the tile for
 // the lane's query row: a ones-row times P^T on the matrix core, from the same
 // bf16 probabilities as the numerator.
+template <bool F16>
 __device__ __forceinline__ void accumulate_tile(lds_ptr vt, const bf16x8 (&pb)[kGroups],
                                                 f32x4 (&acc)[kGroups][8], f32x4 (&lacc)[kGroups], int r,
                                                 int kg) {
@@ -203,14 +229,14 @@ __device__ __forceinline__ void accumulate_tile(lds_ptr vt, const bf16x8 (&pb)[k
         reinterpret_cast<__attribute__((address_space(3))) bf16x4*>(vt + at + 16 * 256));
     va[jd] = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
   }
-  const uint32_t one2 = 0x3F803F80u;   // two bf16 ones
+  const uint32_t one2 = Elem<F16>::kOnes;
   const bf16x8 ones = as_bf16x8(make_uint4(one2, one2, one2, one2));
 #pragma unroll
   for (int g = 0; g < kGroups; ++g) {
-    lacc[g] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ones, pb[g], lacc[g], 0, 0, 0);
+    lacc[g] = Elem<F16>::mfma(ones, pb[g], lacc[g]);
 #pragma unroll
     for (int jd = 0; jd < 8; ++jd)
-      acc[g][jd] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(va[jd], pb[g], acc[g][jd], 0, 0, 0);
+      acc[g][jd] = Elem<F16>::mfma(va[jd], pb[g], acc[g][jd]);
   }
 }
 
@@ -221,7 +247,7 @@ __device__ __forceinline__ void accumulate_tile(lds_ptr vt, const bf16x8 (&pb)[k
 // the sequence), both relative to the first key of the tile, weigh exactly 0.
 // Must run after the previous tile has been accumulated: moving the reference
 // point rescales acc and lacc.
-template <bool MASK>
+template <bool MASK, bool F16>
 __device__ __forceinline__ void probabilities_of_tile(f32x4 (&sc)[kGroups][2], bf16x8 (&pb)[kGroups],
                                                       f32x4 (&acc)[kGroups][8], f32x4 (&lacc)[kGroups],
                                                       float (&m_run)[kGroups], float (&mneg)[kGroups],
@@ -275,10 +301,10 @@ __device__ __forceinline__ void probabilities_of_tile(f32x4 (&sc)[kGroups][2], b
       }
     }
     uint4 pbits;
-    pbits.x = pack_bf16x2(p0[0], p0[1]);
-    pbits.y = pack_bf16x2(p0[2], p0[3]);
-    pbits.z = pack_bf16x2(p1[0], p1[1]);
-    pbits.w = pack_bf16x2(p1[2], p1[3]);
+    pbits.x = Elem<F16>::pack2(p0[0], p0[1]);
+    pbits.y = Elem<F16>::pack2(p0[2], p0[3]);
+    pbits.z = Elem<F16>::pack2(p1[0], p1[1]);
+    pbits.w = Elem<F16>::pack2(p1[2], p1[3]);
     pb[g] = as_bf16x8(pbits);
   }
 }
@@ -295,6 +321,7 @@ struct PrefillArgs {
 };
 
 // grid.x = 8 * ceil(tile bound * Hq / 8) workgroups (see the work-item mapping below).
+template <bool F16>
 __global__ __launch_bounds__(kWaves * 64, kGroups <= 2 ? 2 : 1) void prefill_attention_kernel(PrefillArgs a,
                                                                         int num_tiles_bound) {
   __shared__ uint4 k_ring[kKStages * kTileBytes / 16];
@@ -430,22 +457,22 @@ __global__ __launch_bounds__(kWaves * 64, kGroups <= 2 ? 2 : 1) void prefill_att
   for (int g = 0; g < kGroups; ++g) pb[g] = as_bf16x8(make_uint4(0u, 0u, 0u, 0u));
   int i = 0;
   for (; i < n_plain; ++i) {
-    scores_of_tile(k_lds + k_stage * kTileBytes, qreg, sc, r, kg);
-    accumulate_tile(NVJ_V_BEFORE(), pb, acc, lacc, r, kg);
-    probabilities_of_tile<false>(sc, pb, acc, lacc, m_run, mneg, sl2, r, kg, 0, 0);
+    scores_of_tile<F16>(k_lds + k_stage * kTileBytes, qreg, sc, r, kg);
+    accumulate_tile<F16>(NVJ_V_BEFORE(), pb, acc, lacc, r, kg);
+    probabilities_of_tile<false, F16>(sc, pb, acc, lacc, m_run, mneg, sl2, r, kg, 0, 0);
     NVJ_NEXT_TILE(i);
   }
   for (; i < n_active; ++i) {
     const int ks = i * kKeys;
-    scores_of_tile(k_lds + k_stage * kTileBytes, qreg, sc, r, kg);
-    accumulate_tile(NVJ_V_BEFORE(), pb, acc, lacc, r, kg);
-    probabilities_of_tile<true>(sc, pb, acc, lacc, m_run, mneg, sl2, r, kg, wave_row0 - ks,
+    scores_of_tile<F16>(k_lds + k_stage * kTileBytes, qreg, sc, r, kg);
+    accumulate_tile<F16>(NVJ_V_BEFORE(), pb, acc, lacc, r, kg);
+    probabilities_of_tile<true, F16>(sc, pb, acc, lacc, m_run, mneg, sl2, r, kg, wave_row0 - ks,
                                 k_end - 1 - ks);
     NVJ_NEXT_TILE(i);
   }
   // the last tile of the wave is still to be accumulated; its V stays in place
   // until the copies of two iterations from now
-  if (n_active > 0) accumulate_tile(NVJ_V_BEFORE(), pb, acc, lacc, r, kg);
+  if (n_active > 0) accumulate_tile<F16>(NVJ_V_BEFORE(), pb, acc, lacc, r, kg);
   for (; i < nsteps; ++i) NVJ_NEXT_TILE(i);
   wait_tiles_in_flight<0>();   // copies past the last tile are still landing in LDS
 #undef NVJ_NEXT_TILE
@@ -463,8 +490,8 @@ __global__ __launch_bounds__(kWaves * 64, kGroups <= 2 ? 2 : 1) void prefill_att
 #pragma unroll
       for (int jd = 0; jd < 8; ++jd) {
         uint2 o;
-        o.x = pack_bf16x2(acc[g][jd][0] * inv, acc[g][jd][1] * inv);
-        o.y = pack_bf16x2(acc[g][jd][2] * inv, acc[g][jd][3] * inv);
+        o.x = Elem<F16>::pack2(acc[g][jd][0] * inv, acc[g][jd][1] * inv);
+        o.y = Elem<F16>::pack2(acc[g][jd][2] * inv, acc[g][jd][3] * inv);
         orow[4 * jd + kg] = o;
       }
     }
@@ -478,7 +505,8 @@ extern "C" int nvj_prefill_attention_launch(void* stream, const void* q, const v
                                             const int32_t* cu_seqlens_k, void* out,
                                             int32_t total_q_tokens, int32_t batch,
                                             int32_t num_heads, int32_t num_kv_heads,
-                                            int32_t head_dim, float scale) {
+                                            int32_t head_dim, float scale, int32_t dtype) {
+  if (dtype != NVJ_DTYPE_BF16 && dtype != NVJ_DTYPE_F16) return NVJ_ERR_BAD_DTYPE;
   if (total_q_tokens < 0 || batch < 0 || num_heads <= 0 || num_kv_heads <= 0)
     return NVJ_ERR_BAD_SHAPE;
   if (num_heads % num_kv_heads != 0) return NVJ_ERR_BAD_SHAPE;
@@ -508,7 +536,10 @@ extern "C" int nvj_prefill_attention_launch(void* stream, const void* q, const v
   const int64_t items = tiles * num_heads;
   if (items > INT32_MAX - 8) return NVJ_ERR_BAD_SHAPE;
   const unsigned grid = (unsigned)((items + 7) / 8 * 8);
-  prefill_attention_kernel<<<dim3(grid), dim3(kWaves * 64), 0,
-                             static_cast<hipStream_t>(stream)>>>(a, (int)tiles);
+  const auto hs = static_cast<hipStream_t>(stream);
+  if (dtype == NVJ_DTYPE_F16)
+    prefill_attention_kernel<true><<<dim3(grid), dim3(kWaves * 64), 0, hs>>>(a, (int)tiles);
+  else
+    prefill_attention_kernel<false><<<dim3(grid), dim3(kWaves * 64), 0, hs>>>(a, (int)tiles);
   return hipGetLastError() == hipSuccess ? NVJ_OK : NVJ_ERR_LAUNCH;
 }

@@ -112,7 +112,7 @@ class Attention:
     def _prefill_attention(self, q, k, v, context: AttentionContext):
         """Variable-length causal attention over the packed prompt rows
         (layers/attention.py:331-364)."""
-        dt = torch.bfloat16
+        dt = self.k_cache.dtype           # the model dtype: bf16 or float16
         return variable_length_attention_prefill(
             q.to(dt).contiguous(), k.to(dt).contiguous(), v.to(dt).contiguous(),
             context.cu_seqlens_q, context.cu_seqlens_k, context.max_seqlen_q,

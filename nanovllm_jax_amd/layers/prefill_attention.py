@@ -14,6 +14,8 @@ from .. import _lib
 
 __all__ = ["variable_length_attention_prefill"]
 
+_DTYPE_CODE = {torch.bfloat16: _lib.NVJ_DTYPE_BF16, torch.float16: _lib.NVJ_DTYPE_F16}
+
 
 def _require(cond: bool, msg: str) -> None:
     if not cond:
@@ -24,12 +26,14 @@ def variable_length_attention_prefill(q, k, v, cu_seqlens_q, cu_seqlens_k, max_s
                                       max_seqlen_k=0, num_heads=None, num_kv_heads=None,
                                       scale=None, batch_size=None, *, out=None):
     """q [total_tokens, num_heads, head_dim], k/v [total_k_tokens, num_kv_heads,
-    head_dim] bf16 packed rows; cu_seqlens_q / cu_seqlens_k [batch + 1] int32 on
-    the device.  Query position p of a sequence attends key positions <= p of the
-    same sequence.  Returns [total_tokens, num_heads, head_dim] bf16."""
+    head_dim] packed rows, all bf16 or all float16; cu_seqlens_q / cu_seqlens_k
+    [batch + 1] int32 on the device.  Query position p of a sequence attends key
+    positions <= p of the same sequence.  Returns [total_tokens, num_heads,
+    head_dim] in q's dtype."""
     lib = _lib.load()
-    for name, t, dt, nd in (("q", q, torch.bfloat16, 3), ("k", k, torch.bfloat16, 3),
-                            ("v", v, torch.bfloat16, 3),
+    _require(isinstance(q, torch.Tensor) and q.dtype in _DTYPE_CODE,
+             "q must be a bf16 or float16 torch.Tensor")
+    for name, t, dt, nd in (("q", q, q.dtype, 3), ("k", k, q.dtype, 3), ("v", v, q.dtype, 3),
                             ("cu_seqlens_q", cu_seqlens_q, torch.int32, 1),
                             ("cu_seqlens_k", cu_seqlens_k, torch.int32, 1)):
         _require(isinstance(t, torch.Tensor), f"{name} must be a torch.Tensor")
@@ -51,12 +55,13 @@ def variable_length_attention_prefill(q, k, v, cu_seqlens_q, cu_seqlens_k, max_s
     if out is None:
         out = torch.empty_like(q)
     else:
-        _require(out.is_cuda and out.dtype == torch.bfloat16 and out.shape == q.shape
+        _require(out.is_cuda and out.dtype == q.dtype and out.shape == q.shape
                  and out.is_contiguous(), "out must match q")
     with torch.cuda.device(q.device):
         stream = torch.cuda.current_stream(q.device).cuda_stream
         code = lib.nvj_prefill_attention_launch(
             stream, q.data_ptr(), k.data_ptr(), v.data_ptr(), cu_seqlens_q.data_ptr(),
-            cu_seqlens_k.data_ptr(), out.data_ptr(), total, batch, hq, hkv, d, float(scale))
+            cu_seqlens_k.data_ptr(), out.data_ptr(), total, batch, hq, hkv, d, float(scale),
+            _DTYPE_CODE[q.dtype])
     _lib.check(code, "nvj_prefill_attention_launch")
     return out

@@ -516,7 +516,7 @@ def advance_decode_ref(next_tokens, input_ids, positions, context_lens, slot_map
 # ---------------------------------------------------------------------------
 
 def variable_length_attention_prefill_ref(q, k, v, cu_seqlens_q, cu_seqlens_k, scale,
-                                          return_f32: bool = False):
+                                          return_f32: bool = False, dtype: str = "bf16"):
     """Restates ``variable_length_attention_prefill`` (``layers/attention.py:135-279``)
     without its padding: for sequence i, q rows [cu_q[i], cu_q[i+1]) attend k/v
     rows [cu_k[i], cu_k[i+1]) under ``q_pos >= k_pos`` (:232-236, positions counted
@@ -528,7 +528,9 @@ def variable_length_attention_prefill_ref(q, k, v, cu_seqlens_q, cu_seqlens_k, s
     bf16 result; GQA by head broadcast (h -> h // G).  A query row with no
     visible key is not defined by the reference; zeros here.
 
-    q [T, Hq, D], k/v [Tk, Hkv, D] bf16 bits.  Returns [T, Hq, D] bf16 bits."""
+    q [T, Hq, D], k/v [Tk, Hkv, D] bit patterns of ``dtype`` ("bf16" or "f16").
+    Returns [T, Hq, D] bits of the same type."""
+    decode, encode = _codec(dtype)
     q = np.asarray(q)
     T, Hq, D = q.shape
     Hkv = k.shape[1]
@@ -541,19 +543,19 @@ def variable_length_attention_prefill_ref(q, k, v, cu_seqlens_q, cu_seqlens_k, s
         lq, lk = int(cu_q[i + 1] - cu_q[i]), int(cu_k[i + 1] - cu_k[i])
         if lq <= 0 or lk <= 0:
             continue
-        qs = bf16_bits_to_f32(q[cu_q[i]:cu_q[i + 1]]).reshape(lq, Hkv, G, D)
-        ks = bf16_bits_to_f32(k[cu_k[i]:cu_k[i + 1]])
-        vs = bf16_bits_to_f32(v[cu_k[i]:cu_k[i + 1]])
+        qs = decode(q[cu_q[i]:cu_q[i + 1]]).reshape(lq, Hkv, G, D)
+        ks = decode(k[cu_k[i]:cu_k[i + 1]])
+        vs = decode(v[cu_k[i]:cu_k[i + 1]])
         mask = np.arange(lq)[:, None] >= np.arange(lk)[None, :]           # :232-236
         s = np.einsum("qhgd,khd->hgqk", qs, ks, dtype=np.float32) * scale
         s = np.where(mask[None, None], s, np.float32(-1e30))
         s = s - s.max(axis=-1, keepdims=True)
         e = np.where(mask[None, None], np.exp(s, dtype=np.float32), np.float32(0))
         p = e / e.sum(axis=-1, keepdims=True, dtype=np.float32)
-        p = bf16_bits_to_f32(f32_to_bf16_bits(p))                         # probs -> value dtype
+        p = decode(encode(p))                                            # probs -> value dtype
         o = np.einsum("hgqk,khd->qhgd", p, vs, dtype=np.float32)
         out[cu_q[i]:cu_q[i + 1]] = o.reshape(lq, Hq, D)
-    return out if return_f32 else f32_to_bf16_bits(out)
+    return out if return_f32 else encode(out)
 
 
 def textbook_prefill_f64(q, k, v, cu_seqlens_q, cu_seqlens_k, scale):

@@ -96,3 +96,98 @@ def test_mixed_dtypes_are_refused():
     with pytest.raises(ValueError):
         store_kv_to_cache(k, k, kc.view(-1, 8, 128), kc.view(-1, 8, 128),
                           torch.zeros(1, dtype=torch.int32, device=dev))   # f16 rows, bf16 cache
+
+
+def test_prefill_float16():
+    print("case f16 prefill", flush=True)
+    import torch
+    from nanovllm_jax_amd import variable_length_attention_prefill
+    from nanovllm_jax_amd.workloads import draw_bf16_bits
+    from oracle.paged_attention_oracle import (bf16_bits_to_f32, f16_bits_to_f32, f32_to_f16_bits,
+                                               variable_length_attention_prefill_ref)
+    rng = np.random.Generator(np.random.PCG64(830))
+    lens = [1, 33, 128, 300, 0, 517]
+    Hq, Hkv, D = 16, 4, 128
+    cu = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
+    cv = lambda b: f32_to_f16_bits(bf16_bits_to_f32(b) * np.float32(1.001))
+    q = cv(draw_bf16_bits(rng, (int(cu[-1]), Hq, D), 2.0))
+    k = cv(draw_bf16_bits(rng, (int(cu[-1]), Hkv, D)))
+    v = cv(draw_bf16_bits(rng, (int(cu[-1]), Hkv, D)))
+    dev = "cuda:0"
+    scale = D ** -0.5
+    out = variable_length_attention_prefill(_to_f16(q, dev), _to_f16(k, dev), _to_f16(v, dev),
+                                            torch.from_numpy(cu).to(dev),
+                                            torch.from_numpy(cu).to(dev), scale=scale)
+    torch.cuda.synchronize()
+    assert out.dtype == torch.float16
+    got = f16_bits_to_f32(_bits(out)).astype(np.float64)
+    want = f16_bits_to_f32(variable_length_attention_prefill_ref(q, k, v, cu, cu, scale,
+                                                                 dtype="f16")).astype(np.float64)
+    err = np.abs(got - want)
+    assert np.all(err <= 1e-2 + 1e-2 * np.abs(want)), f"max err {err.max():.3e}"
+    assert np.array_equal(got[0], np.repeat(f16_bits_to_f32(v[0]), Hq // Hkv, axis=0))  # 1 key
+
+
+def test_attention_layer_with_float16_caches_prefill_then_decode():
+    """The layer call of the reference (layers/attention.py:436-480) on a float16
+    model: store + prefill attention, then store + decode attention over the
+    same cache, every result float16."""
+    print("case f16 Attention layer prefill then decode", flush=True)
+    import torch
+    from nanovllm_jax_amd import Attention, create_decode_context, create_prefill_context
+    from nanovllm_jax_amd.workloads import draw_bf16_bits
+    from oracle.paged_attention_oracle import (bf16_bits_to_f32, f16_bits_to_f32, f32_to_f16_bits,
+                                               paged_decode_attention_per_seq_ref,
+                                               store_kv_to_cache_ref,
+                                               variable_length_attention_prefill_ref)
+    rng = np.random.Generator(np.random.PCG64(840))
+    Hq, Hkv, D, bs, NB = 8, 2, 128, 64, 12
+    lens = [70, 5, 129]
+    B = len(lens)
+    cu = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
+    T = int(cu[-1])
+    cv = lambda b: f32_to_f16_bits(bf16_bits_to_f32(b))
+    q, k, v = (cv(draw_bf16_bits(rng, (T, h, D))) for h in (Hq, Hkv, Hkv))
+    pages = rng.permutation(NB)
+    bt = np.full((B, 3), -1, np.int32)
+    slots = np.zeros(T, np.int32)
+    used = 0
+    for b, n in enumerate(lens):
+        nb = -(-n // bs)
+        bt[b, :nb] = pages[used:used + nb]
+        used += nb
+        pos = np.arange(n)
+        slots[cu[b]:cu[b + 1]] = bt[b, pos // bs] * bs + pos % bs
+    dev = "cuda:0"
+    kc = torch.zeros((NB, bs, Hkv, D), dtype=torch.float16, device=dev)
+    vc = torch.zeros_like(kc)
+    attn = Attention(Hq, D, D ** -0.5, Hkv, bs)
+    attn.set_kv_cache(kc, vc)
+    ctx = create_prefill_context(torch.from_numpy(cu).to(dev), torch.from_numpy(cu).to(dev),
+                                 max(lens), max(lens), torch.from_numpy(slots).to(dev))
+    out = attn(_to_f16(q, dev), _to_f16(k, dev), _to_f16(v, dev), ctx)
+    torch.cuda.synchronize()
+    assert out.dtype == torch.float16
+    want = variable_length_attention_prefill_ref(q, k, v, cu, cu, D ** -0.5, dtype="f16")
+    err = np.abs(f16_bits_to_f32(_bits(out)).astype(np.float64) - f16_bits_to_f32(want))
+    assert np.all(err <= 1e-2 + 1e-2 * np.abs(f16_bits_to_f32(want))), f"prefill {err.max():.3e}"
+    flat = (NB * bs, Hkv, D)
+    zero = np.zeros(flat, np.uint16)
+    wk, wv = store_kv_to_cache_ref(k, v, zero, zero.copy(), slots, negative_slots="skip",
+                                   dtype="f16")
+    assert np.array_equal(_bits(kc).reshape(flat), wk) and np.array_equal(_bits(vc).reshape(flat), wv)
+    # one decode step on top
+    q1, k1, v1 = (cv(draw_bf16_bits(rng, (B, h, D))) for h in (Hq, Hkv, Hkv))
+    new_len = np.array(lens, np.int32) + 1
+    slot1 = np.array([bt[b, (n - 1) // bs] * bs + (n - 1) % bs for b, n in enumerate(new_len)],
+                     np.int32)
+    dctx = create_decode_context(torch.from_numpy(new_len).to(dev), torch.from_numpy(slot1).to(dev),
+                                 torch.from_numpy(bt).to(dev))
+    out1 = attn(_to_f16(q1, dev), _to_f16(k1, dev), _to_f16(v1, dev), dctx)
+    torch.cuda.synchronize()
+    wk, wv = store_kv_to_cache_ref(k1, v1, wk, wv, slot1, negative_slots="skip", dtype="f16")
+    want1 = paged_decode_attention_per_seq_ref(q1, wk.reshape(NB, bs, Hkv, D),
+                                               wv.reshape(NB, bs, Hkv, D), bt, new_len, D ** -0.5,
+                                               bs, dtype="f16")
+    err = np.abs(f16_bits_to_f32(_bits(out1)).astype(np.float64) - f16_bits_to_f32(want1))
+    assert np.all(err <= 1e-2 + 1e-2 * np.abs(f16_bits_to_f32(want1))), f"decode {err.max():.3e}"
