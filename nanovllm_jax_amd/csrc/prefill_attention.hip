@@ -456,18 +456,26 @@ __global__ __launch_bounds__(kWaves * 64, kGroups <= 2 ? 2 : 1) void prefill_att
 #pragma unroll
   for (int g = 0; g < kGroups; ++g) pb[g] = as_bf16x8(make_uint4(0u, 0u, 0u, 0u));
   int i = 0;
+  // Waves that issue matrix instructions go first: a wave lowers its priority
+  // only while it turns scores into probabilities (vector ALU work that the
+  // other wave of the SIMD can overlap with its own matrix instructions).
+  __builtin_amdgcn_s_setprio(1);
   for (; i < n_plain; ++i) {
     scores_of_tile<F16>(k_lds + k_stage * kTileBytes, qreg, sc, r, kg);
     accumulate_tile<F16>(NVJ_V_BEFORE(), pb, acc, lacc, r, kg);
+    __builtin_amdgcn_s_setprio(0);
     probabilities_of_tile<false, F16>(sc, pb, acc, lacc, m_run, mneg, sl2, r, kg, 0, 0);
+    __builtin_amdgcn_s_setprio(1);
     NVJ_NEXT_TILE(i);
   }
   for (; i < n_active; ++i) {
     const int ks = i * kKeys;
     scores_of_tile<F16>(k_lds + k_stage * kTileBytes, qreg, sc, r, kg);
     accumulate_tile<F16>(NVJ_V_BEFORE(), pb, acc, lacc, r, kg);
+    __builtin_amdgcn_s_setprio(0);
     probabilities_of_tile<true, F16>(sc, pb, acc, lacc, m_run, mneg, sl2, r, kg, wave_row0 - ks,
                                 k_end - 1 - ks);
+    __builtin_amdgcn_s_setprio(1);
     NVJ_NEXT_TILE(i);
   }
   // the last tile of the wave is still to be accumulated; its V stays in place
