@@ -434,10 +434,26 @@ __device__ __forceinline__ void compute_segment_valu(const DecodeArgs& a, uint4*
   float* lds_ml = lds_o + G * D;
   static_assert((512 + 8 * 128 + 16) * 4 <= kStep * H::kLdsRowPieces * 16, "fits the K tile");
 
-  uint4 qv[G];   // dims 8*r .. +8 of every query row of the group
+  // dims 8*r .. +8 of every query row of the group: in registers up to 4 rows,
+  // in the wave's LDS tile beyond (read back per batch, the same address in
+  // the four lanes that share r), which keeps the 8-row form free of spills
+  constexpr bool kQInLds = G > 4;
+  uint4* lds_q = lds + 400;   // byte 6400, behind the hand-over area; G * 16 pieces
+  static_assert(400 + 8 * 16 <= kStep * H::kLdsRowPieces, "q pieces fit the K tile");
+  uint4 qv[kQInLds ? 1 : G];
+  if constexpr (kQInLds) {
 #pragma unroll
-  for (int h = 0; h < G; ++h)
-    qv[h] = a.q[((int64_t)b * a.num_heads + (int64_t)kvh * G + h) * H::kPieces + r];
+    for (int h = kg; h < G; h += 4)
+      lds_q[h * H::kPieces + r] =
+          a.q[((int64_t)b * a.num_heads + (int64_t)kvh * G + h) * H::kPieces + r];
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+  } else {
+#pragma unroll
+    for (int h = 0; h < G; ++h)
+      qv[h] = a.q[((int64_t)b * a.num_heads + (int64_t)kvh * G + h) * H::kPieces + r];
+  }
 
   // the scores this lane owns after the exchange: entry c of a batch is partial
   // index n = low + 16 * c, low = the bits of r in reverse order; n = h + G * i
@@ -497,10 +513,11 @@ __device__ __forceinline__ void compute_segment_valu(const DecodeArgs& a, uint4*
 #pragma unroll
         for (int h = 0; h < G; ++h) {
           const uint4 kk = kreg[bt * LB + i];
-          float s = dot2_bf16(kk.x, qv[h].x, 0.f);
-          s = dot2_bf16(kk.y, qv[h].y, s);
-          s = dot2_bf16(kk.z, qv[h].z, s);
-          part[h + G * i] = dot2_bf16(kk.w, qv[h].w, s);
+          const uint4 qq = kQInLds ? lds_q[h * H::kPieces + r] : qv[kQInLds ? 0 : h];
+          float s = dot2_bf16(kk.x, qq.x, 0.f);
+          s = dot2_bf16(kk.y, qq.y, s);
+          s = dot2_bf16(kk.z, qq.z, s);
+          part[h + G * i] = dot2_bf16(kk.w, qq.w, s);
         }
       halve_across<kDppRowMirror, NB / 2>(part, (r & 8) != 0);
       halve_across<kDppHalfMirror, NB / 4>(part, (r & 4) != 0);
