@@ -85,5 +85,22 @@ def build_xla_ffi(verbose: bool = True) -> str | None:
     return out
 
 
+def build_c_caller(verbose: bool = True) -> str:
+    """Compile the plain-C caller of the C ABI (csrc/c_caller) with the host C
+    compiler against the library just built; the GPU tests run it as a child
+    process to show the ABI needs neither C++ nor torch on the calling side."""
+    out = os.path.join(NATIVE_DIR, "nvj_c_caller")
+    rocm = os.environ.get("ROCM_PATH", "/opt/rocm")
+    cmd = [os.environ.get("CC", "gcc"), "-std=c11", "-O2", "-Wall", "-Wextra",
+           "-I", os.path.join(REPO_DIR, "include"), "-I", os.path.join(rocm, "include"),
+           os.path.join(CSRC_DIR, "c_caller", "nvj_c_caller.c"),
+           "-L", NATIVE_DIR, "-lnvj_paged_attn", "-L", os.path.join(rocm, "lib"), "-lamdhip64",
+           "-Wl,-rpath,$ORIGIN", "-Wl,-rpath," + os.path.join(rocm, "lib"), "-o", out]
+    if verbose:
+        print("[build]", " ".join(cmd), flush=True)
+    subprocess.run(cmd, check=True)
+    return out
+
+
 if __name__ == "__main__":
     print(build(extra_flags=tuple(sys.argv[1:])))
