@@ -244,15 +244,16 @@ __device__ __forceinline__ void compute_segment(const DecodeArgs& a, uint4* lds,
   m_run = kNegBig;  // running max of raw scores (q.k, unscaled) of column r
   l_run = 0.f;      // this lane's share of the running sum
 
+  // the page lookup of a step is started two steps ahead, so that its latency
+  // is not in front of the loads that need the address
+  int64_t off_ahead = nsteps > 1 ? step_base(1) : 0;
   for (int step = 0; step < nsteps; ++step) {
     const int nvalid = min(kStep, t1 - (t0 + step * kStep));
     const bool more = step + 1 < nsteps;
-    int64_t next_off = 0;
+    const int64_t next_off = off_ahead;
     int next_last = kStep - 1;
-    if (more) {
-      next_off = step_base(step + 1);
-      next_last = min(kStep, t1 - (t0 + (step + 1) * kStep)) - 1;
-    }
+    if (more) next_last = min(kStep, t1 - (t0 + (step + 1) * kStep)) - 1;
+    if (step + 2 < nsteps) off_ahead = step_base(step + 2);
 
     // ---- K: registers -> LDS (row = position, padded), then next K loads ----
 #pragma unroll
@@ -493,15 +494,16 @@ __device__ __forceinline__ void compute_segment_valu(const DecodeArgs& a, uint4*
     for (int jd = 0; jd < 8; ++jd) acc[h][jd] = 0.f;
   float m_run = kNegBig, l_run = 0.f;   // of head my_h; l_run is this lane's share
 
+  // the page lookup of a step is started two steps ahead, so that its latency
+  // is not in front of the loads that need the address
+  int64_t off_ahead = nsteps > 1 ? step_base(1) : 0;
   for (int step = 0; step < nsteps; ++step) {
     const int nvalid = min(kStep, t1 - (t0 + step * kStep));
     const bool more = step + 1 < nsteps;
-    int64_t next_off = 0;
+    const int64_t next_off = off_ahead;
     int next_last = kStep - 1;
-    if (more) {
-      next_off = step_base(step + 1);
-      next_last = min(kStep, t1 - (t0 + (step + 1) * kStep)) - 1;
-    }
+    if (more) next_last = min(kStep, t1 - (t0 + (step + 1) * kStep)) - 1;
+    if (step + 2 < nsteps) off_ahead = step_base(step + 2);
 
     // ---- scores, batch by batch, then next K loads ----
     float v[NS];
