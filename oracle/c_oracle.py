@@ -27,10 +27,12 @@ def _load():
         lib = ctypes.CDLL(_SO)
         lib.oracle_num_threads.restype = ctypes.c_int
         lib.oracle_paged_decode.restype = ctypes.c_int
-        lib.oracle_paged_decode.argtypes = [ctypes.c_void_p] * 7 + [ctypes.c_int] * 7 + [ctypes.c_float]
+        lib.oracle_paged_decode.argtypes = ([ctypes.c_void_p] * 7 + [ctypes.c_int] * 7 +
+                                            [ctypes.c_float, ctypes.c_int])
         lib.oracle_store_kvcache.restype = None
         lib.oracle_store_kvcache.argtypes = ([ctypes.c_void_p] * 5 + [ctypes.c_int, ctypes.c_int,
-                                             ctypes.c_int64, ctypes.c_int, ctypes.c_int, ctypes.c_int])
+                                             ctypes.c_int64, ctypes.c_int, ctypes.c_int, ctypes.c_int,
+                                             ctypes.c_int])
         _lib = lib
     return _lib
 
@@ -44,8 +46,9 @@ def _ptr(a):
 
 
 def paged_decode(q, k_cache, v_cache, block_tables, context_lens, scale, block_size,
-                 return_f32=False):
+                 return_f32=False, dtype="bf16"):
     """Same contract as ``paged_decode_attention_per_seq_ref``."""
+    assert dtype in ("bf16", "f16")
     lib = _load()
     q = np.ascontiguousarray(q, np.uint16)
     kc = np.ascontiguousarray(k_cache, np.uint16)
@@ -59,13 +62,15 @@ def paged_decode(q, k_cache, v_cache, block_tables, context_lens, scale, block_s
     of = np.empty((B, Hq, D), np.float32)
     ob = np.empty((B, Hq, D), np.uint16)
     rc = lib.oracle_paged_decode(_ptr(q), _ptr(kc), _ptr(vc), _ptr(bt), _ptr(ctx), _ptr(of),
-                                 _ptr(ob), B, Hq, Hkv, D, bs, MB, NB, float(scale))
+                                 _ptr(ob), B, Hq, Hkv, D, bs, MB, NB, float(scale),
+                                 int(dtype == "f16"))
     if rc != 0:
         raise RuntimeError("oracle_paged_decode: unsupported sizes")
     return of if return_f32 else ob
 
 
-def store_kvcache(key, value, k_cache, v_cache, slot_mapping, negative_slots="reference"):
+def store_kvcache(key, value, k_cache, v_cache, slot_mapping, negative_slots="reference",
+                  dtype="bf16"):
     """Same contract as ``store_kv_to_cache_ref`` (returns new caches)."""
     lib = _load()
     key = np.ascontiguousarray(key)
@@ -78,5 +83,5 @@ def store_kvcache(key, value, k_cache, v_cache, slot_mapping, negative_slots="re
     lib.oracle_store_kvcache(_ptr(key), _ptr(value), _ptr(kc), _ptr(vc), _ptr(slots), T, row,
                              kc.shape[0], int(key.dtype == np.float32),
                              int(value.dtype == np.float32),
-                             1 if negative_slots == "skip" else 0)
+                             1 if negative_slots == "skip" else 0, int(dtype == "f16"))
     return kc, vc

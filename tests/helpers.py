@@ -17,7 +17,7 @@ def bits_to_torch(bits: np.ndarray, device="cpu"):
 
 def torch_to_bits(t) -> np.ndarray:
     import torch
-    assert t.dtype == torch.bfloat16
+    assert t.dtype in (torch.bfloat16, torch.float16)
     return t.detach().cpu().contiguous().view(torch.int16).numpy().view(np.uint16).copy()
 
 

@@ -17,7 +17,7 @@ if ROOT not in sys.path:
 pytestmark = pytest.mark.gpu
 
 
-def _run(name, chunks):
+def _run(name, chunks, dtype="bf16"):
     import torch
     import bench
     from nanovllm_jax_amd import paged_attention
@@ -25,7 +25,8 @@ def _run(name, chunks):
     from oracle import c_oracle
     dev = torch.device("cuda:0")
     w = make_workload(name)
-    q, kc, vc, bt, ctx, slots, k_new, v_new = bench.device_inputs(w, torch, dev)
+    dt = torch.float16 if dtype == "f16" else torch.bfloat16
+    q, kc, vc, bt, ctx, slots, k_new, v_new = bench.device_inputs(w, torch, dev, dt)
     outs = []
     for ch in chunks:
         print(f"case {name} full size chunk={ch}", flush=True)
@@ -33,9 +34,16 @@ def _run(name, chunks):
         torch.cuda.synchronize()
         outs.append(torch_to_bits(out))
     want = c_oracle.paged_decode(torch_to_bits(q), torch_to_bits(kc), torch_to_bits(vc),
-                                 w.block_tables, w.context_lens, w.scale, w.block_size)
+                                 w.block_tables, w.context_lens, w.scale, w.block_size,
+                                 dtype=dtype)
     for ch, got in zip(chunks, outs):
-        err = assert_close_bf16(got, want, what=f"{name} chunk={ch}")
+        if dtype == "f16":
+            from oracle.paged_attention_oracle import f16_bits_to_f32
+            g, t = (f16_bits_to_f32(a).astype(np.float64) for a in (got, want))
+            assert np.all(np.abs(g - t) <= 1e-2 + 1e-2 * np.abs(t)), f"{name} f16 chunk={ch}"
+            err = float(np.abs(g - t).max())
+        else:
+            err = assert_close_bf16(got, want, what=f"{name} chunk={ch}")
         print(f"  {name} chunk={ch}: max abs err {err:.3e}", flush=True)
     del q, kc, vc
     torch.cuda.empty_cache()
@@ -44,6 +52,10 @@ def _run(name, chunks):
 
 def test_c2_qwen3_8b_shape():
     _run("C2", [0, 256])
+
+
+def test_c2_float16_caches():
+    _run("C2", [0, -1], dtype="f16")
 
 
 def test_c5_layer_shape():

@@ -458,3 +458,43 @@ def test_f16_rounding_against_torch_and_special_values():
     assert f32_to_f16_bits(np.array([65520.0], np.float32))[0] == 0x7C00
     all_bits = np.arange(0x7C00, dtype=np.uint16)
     assert np.array_equal(f32_to_f16_bits(f16_bits_to_f32(all_bits)), all_bits)
+
+
+def test_c_oracle_float16_matches_the_numpy_restatement():
+    """The C restatement with IEEE-half elements: store bit for bit (its f32 -> half
+    rounding over subnormals, ties, overflow and NaN), decode within float32
+    round-off of the NumPy restatement, same rounded output except at ties."""
+    from oracle.paged_attention_oracle import (f16_bits_to_f32, f32_to_f16_bits,
+                                               paged_decode_attention_per_seq_ref,
+                                               store_kv_to_cache_ref)
+    rng = np.random.Generator(np.random.PCG64(77))
+    T, Hkv, D, slots_n = 64, 2, 64, 200
+    vals = (rng.standard_normal((2, T, Hkv, D)) * np.exp(rng.uniform(-20, 12, (2, T, Hkv, D)))
+            ).astype(np.float32)
+    vals[0, 0, 0, :8] = [65504.0, 65520.0, 65519.99, 1e-8, 6.0e-8, 2.98e-8, -0.0, np.nan]
+    kc = rng.integers(0, 0x7C00, (slots_n, Hkv, D)).astype(np.uint16)
+    slots = rng.permutation(slots_n)[:T].astype(np.int32)
+    wk, wv = store_kv_to_cache_ref(vals[0], vals[1], kc, kc.copy(), slots, negative_slots="skip",
+                                   dtype="f16")
+    ck, cv = c_oracle.store_kvcache(vals[0], vals[1], kc, kc.copy(), slots, negative_slots="skip",
+                                    dtype="f16")
+    nan = np.isnan(f16_bits_to_f32(wk))
+    assert np.array_equal(nan, np.isnan(f16_bits_to_f32(ck)))
+    assert np.array_equal(np.where(nan, 0, wk), np.where(nan, 0, ck)) and np.array_equal(wv, cv)
+    # every finite half value decodes to the same float in C: round trip through the store
+    all_bits = np.arange(0x7C00, dtype=np.uint16).reshape(-1, 1, 64)
+    allf = f16_bits_to_f32(all_bits)
+    z = np.zeros_like(all_bits)
+    rk, _ = c_oracle.store_kvcache(allf, allf, z, z.copy(), np.arange(all_bits.shape[0], dtype=np.int32),
+                                   dtype="f16")
+    assert np.array_equal(rk, all_bits)
+    B, Hq, Hkv, D, bs, NB = 5, 8, 2, 128, 64, 24
+    q, kc, vc, bt, ctx = make_problem(78, B, Hq, Hkv, D, bs, NB, [0, 1, 65, 200, 130])
+    cv16 = lambda b: f32_to_f16_bits(bf16_bits_to_f32(b) * np.float32(1.01))
+    q, kc, vc = cv16(q), cv16(kc), cv16(vc)
+    want = paged_decode_attention_per_seq_ref(q, kc, vc, bt, ctx, 0.09, bs, return_f32=True,
+                                              dtype="f16")
+    got = c_oracle.paged_decode(q, kc, vc, bt, ctx, 0.09, bs, return_f32=True, dtype="f16")
+    assert np.allclose(got, want, rtol=1e-5, atol=1e-6)
+    got_bits = c_oracle.paged_decode(q, kc, vc, bt, ctx, 0.09, bs, dtype="f16")
+    assert np.array_equal(got_bits, f32_to_f16_bits(got))
