@@ -170,10 +170,11 @@ def bench_prefill(args, torch):
     (Hq=32, Hkv=8, D=128): 8 prompts of 4096 tokens, packed.  Reports TFLOP/s
     (4 * Hq * D flop per visible (query, key) pair) against the dense bf16 MFMA
     peak."""
-    from nanovllm_jax_amd import variable_length_attention_prefill
+    from nanovllm_jax_amd import paged_prefill_attention, variable_length_attention_prefill
     dev = torch.device("cuda:0")
     hq, hkv, d = 32, 8, 128
     lens = [int(x) for x in args.prefill_lens.split(",")]
+    prefix = int(args.prefill_prefix)
     cu = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
     g = torch.Generator(device=dev)
     g.manual_seed(7)
@@ -184,17 +185,37 @@ def bench_prefill(args, torch):
     cu_t = torch.from_numpy(cu).to(dev)
     out = torch.empty_like(q)
     fn = lambda: variable_length_attention_prefill(q, k, v, cu_t, cu_t, scale=d ** -0.5, out=out)
+    if prefix > 0:
+        # every prompt sits behind `prefix` cached positions: keys and values come
+        # from a paged cache (page 256, pages in random order)
+        bs = 256
+        lens_k = [n + prefix for n in lens]
+        nblk = [-(-n // bs) for n in lens_k]
+        rng = np.random.Generator(np.random.PCG64(7))
+        pages = rng.permutation(sum(nblk))
+        bt = np.full((len(lens), max(nblk)), -1, np.int32)
+        used = 0
+        for i, n in enumerate(nblk):
+            bt[i, :n] = pages[used:used + n]
+            used += n
+        kc = torch.randn((sum(nblk), bs, hkv, d), generator=g, device=dev).to(torch.bfloat16)
+        vc = torch.randn((sum(nblk), bs, hkv, d), generator=g, device=dev).to(torch.bfloat16)
+        cu_k = torch.from_numpy(np.concatenate([[0], np.cumsum(lens_k)]).astype(np.int32)).to(dev)
+        bt_t = torch.from_numpy(bt).to(dev)
+        fn = lambda: paged_prefill_attention(q, kc, vc, bt_t, cu_t, cu_k, d ** -0.5, out=out)
     for _ in range(args.warmup):
         fn()
     ms, wall = timed(fn, args.steps, torch)
-    pairs = sum(n * (n + 1) // 2 for n in lens)
+    pairs = sum(n * (n + 1) // 2 + n * prefix for n in lens)
     flops = 4.0 * hq * d * pairs
     tflops = flops / (ms * 1e-3) / 1e12
     rec = {"metric": "prefill attention TFLOP/s (causal, varlen, Qwen3-8B head shape)",
            "value": round(tflops, 1), "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps,
            "warmup": args.warmup, "ms_per_step": round(wall, 4), "higher_is_better": True,
            "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
-           "config": {"workload": f"prefill: Hq={hq} Hkv={hkv} D={d}, prompt lengths {lens}",
+           "config": {"workload": f"prefill: Hq={hq} Hkv={hkv} D={d}, prompt lengths {lens}" +
+                                  (f" behind {prefix} cached positions each (paged cache)"
+                                   if prefix > 0 else ""),
                       "flops_per_call": flops},
            "roofline": {"bound": "mfma", "achieved": round(tflops, 1),
                         "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
@@ -230,6 +251,9 @@ def main():
                     help="time the prefill attention kernel instead; prints its own JSON line")
     ap.add_argument("--prefill-lens", default=",".join(["4096"] * 8),
                     help="comma-separated prompt lengths for --prefill")
+    ap.add_argument("--prefill-prefix", type=int, default=0,
+                    help="with --prefill: cached positions in front of every prompt; keys and "
+                         "values are then read from a paged cache")
     ap.add_argument("--decode-step", action="store_true",
                     help="time the whole-model decode step (config C5) instead of the "
                          "attention call; prints its own JSON line")

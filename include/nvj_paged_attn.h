@@ -293,6 +293,35 @@ NVJ_API int nvj_prefill_attention_launch(void* stream, const void* q, const void
                             int32_t num_kv_heads, int32_t head_dim, float scale, int32_t dtype);
 
 /*
+ * The same attention with keys and values read from the block-paged cache:
+ * prompt rows behind a cached prefix (prefix caching, chunked prefill).  The
+ * reference prepares exactly this call - cu_seqlens_k > cu_seqlens_q and
+ * block_tables in the prefill context (engine/model_runner.py:286-312,
+ * utils/context.py:129-166) - but its attention (layers/attention.py:331-364)
+ * is handed only the new rows and never reads the cached part; this entry point
+ * is what that context describes.  Run it after the store of the new rows.
+ *
+ *   q   [total_q_tokens, num_heads, head_dim]                     `dtype`
+ *   k_cache, v_cache [num_blocks, block_size, num_kv_heads, head_dim]  `dtype`
+ *   block_tables [batch, max_blocks] int32 (entries of live pages in [0, num_blocks))
+ *   cu_seqlens_q, cu_seqlens_k [batch + 1] int32; len_k = cu_k[i+1] - cu_k[i] counts
+ *       the keys of sequence i, cached and new together (clamped to
+ *       max_blocks * block_size), as the reference's filler sets it (:288-291)
+ *   out [total_q_tokens, num_heads, head_dim]                     `dtype`
+ *
+ * The len_q = cu_q[i+1] - cu_q[i] query rows of sequence i are its LAST len_q
+ * positions: row j attends key positions <= len_k - len_q + j.  With
+ * len_k == len_q this is nvj_prefill_attention_launch on the rows just
+ * stored, bit for bit.  head_dim 128, block_size a multiple of 32, scale >= 0.
+ */
+NVJ_API int nvj_paged_prefill_attention_launch(void* stream, const void* q, const void* k_cache,
+                            const void* v_cache, const int32_t* block_tables,
+                            const int32_t* cu_seqlens_q, const int32_t* cu_seqlens_k, void* out,
+                            int32_t total_q_tokens, int32_t batch, int32_t num_heads,
+                            int32_t num_kv_heads, int32_t head_dim, int32_t block_size,
+                            int32_t max_blocks, int32_t num_blocks, float scale, int32_t dtype);
+
+/*
  * RMSNorm over the last dimension, optionally fused with the residual add.
  * Replaces RMSNorm._rms_forward (layers/layernorm.py:31-48) when `residual` is
  * NULL and RMSNorm._add_rms_forward (layers/layernorm.py:50-79) otherwise, as

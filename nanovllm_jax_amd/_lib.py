@@ -49,6 +49,8 @@ SYMBOLS = {
     "nvj_prefill_attention_launch": (_c.c_int, [
         _c.c_void_p, _c.c_void_p, _c.c_void_p, _c.c_void_p, _c.c_void_p, _c.c_void_p, _c.c_void_p,
         _c.c_int32, _c.c_int32, _c.c_int32, _c.c_int32, _c.c_int32, _c.c_float, _c.c_int32]),
+    "nvj_paged_prefill_attention_launch": (_c.c_int, [
+        _c.c_void_p] * 8 + [_c.c_int32] * 8 + [_c.c_float, _c.c_int32]),
     "nvj_add_rms_norm_launch": (_c.c_int, [
         _c.c_void_p, _c.c_void_p, _c.c_void_p, _c.c_void_p, _c.c_float, _c.c_void_p, _c.c_void_p,
         _c.c_int32, _c.c_int32]),

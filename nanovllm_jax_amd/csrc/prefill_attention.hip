@@ -129,19 +129,33 @@ __device__ __forceinline__ void copy16_to_lds(const char* base, uint32_t offset,
 // k_end is read.
 constexpr int kCopyRowsPerWave = kKeys / kWaves;   // rows of a tile one wave copies
 static_assert(kCopyRowsPerWave % 4 == 0, "one copy instruction covers 4 rows");
+// Packed rows: key s of the sequence is row s behind k_head / v_head.  Paged
+// (PAGED): k_head / v_head point at this kv head inside row 0 of the caches and
+// key s is row table[s / block_size] * block_size + s % block_size; a tile of 32
+// keys never leaves its page (block_size is a multiple of 32), so one scalar
+// table lookup per tile gives the base and the lanes keep their row offsets.
+template <bool PAGED>
 struct TileCopier {
   const char* k_head;   // first key row of the sequence for this kv head
   const char* v_head;
   uint32_t row_bytes;   // bytes between consecutive keys; < 2^24 (checked by the host)
   uint32_t k_lds, v_lds;   // LDS byte addresses of the two rings
   int last_key, last_tile, wave, lane;
+  const_i32_ptr table;  // PAGED: this sequence's row of the block tables
+  int block_size, num_blocks;
 
   __device__ __forceinline__ void issue(int tile, int k_stage, int v_stage) const {
     tile = min(tile, last_tile);   // past the end: fetch the last tile again (same instruction count)
     const int ks = tile * kKeys;
     const int cap = last_key - ks;   // >= 0: a tile starts at a visible key
-    const char* kb = k_head + (size_t)ks * row_bytes;
-    const char* vb = v_head + (size_t)ks * row_bytes;
+    size_t first_row = (size_t)ks;
+    if (PAGED) {
+      const int page = ks / block_size;
+      const int phys = min(max(table[page], 0), num_blocks - 1);
+      first_row = (size_t)phys * block_size + (ks - page * block_size);
+    }
+    const char* kb = k_head + first_row * row_bytes;
+    const char* vb = v_head + first_row * row_bytes;
 #pragma unroll
     for (int j = 0; j < kCopyRowsPerWave / 4; ++j) {
       const int row = kCopyRowsPerWave * wave + 4 * j + (lane >> 4);
@@ -315,13 +329,21 @@ struct PrefillArgs {
   const uint4* v;
   uint4* out;           // [Tq, Hq, 16] pieces
   const int32_t* cu_q;  // [B + 1]
-  const int32_t* cu_k;  // [B + 1]
+  const int32_t* cu_k;  // [B + 1]; paged: the keys of a sequence, cached and new together
   int batch, num_heads, num_kv_heads, group;
   float scale_log2e;
+  // paged only: k and v are the caches [num_blocks, block_size, Hkv, 16] pieces
+  const int32_t* block_tables;   // [B, max_blocks]
+  int block_size, max_blocks, num_blocks;
 };
 
 // grid.x = 8 * ceil(tile bound * Hq / 8) workgroups (see the work-item mapping below).
-template <bool F16>
+// PAGED: keys and values come from the block-paged cache through block_tables,
+// sequence i has len_k = cu_k[i+1] - cu_k[i] keys, and its len_q query rows are the
+// LAST len_q positions of the sequence (row j sees keys <= len_k - len_q + j):
+// prompt rows behind a cached prefix.  Otherwise: packed rows, both counted
+// from the start of the sequence as the reference's mask does.
+template <bool F16, bool PAGED>
 __global__ __launch_bounds__(kWaves * 64, kGroups <= 2 ? 2 : 1) void prefill_attention_kernel(PrefillArgs a,
                                                                         int num_tiles_bound) {
   __shared__ uint4 k_ring[kKStages * kTileBytes / 16];
@@ -368,9 +390,13 @@ __global__ __launch_bounds__(kWaves * 64, kGroups <= 2 ? 2 : 1) void prefill_att
   }
   if (seq < 0) return;   // beyond the real number of tiles
   const int q_base = cu_q[seq], len_q = cu_q[seq + 1] - q_base;
-  const int k_base = cu_k[seq], len_k = max(cu_k[seq + 1] - k_base, 0);
+  const int k_base = PAGED ? 0 : cu_k[seq];
+  const int len_k = PAGED ? min(max(cu_k[seq + 1] - cu_k[seq], 0), a.max_blocks * a.block_size)
+                          : max(cu_k[seq + 1] - k_base, 0);
+  // key position of query row 0: rows are the tail of the sequence when paged
+  const int off = PAGED ? max(len_k - len_q, 0) : 0;
   const int q_end = min(q0 + kBM, len_q);           // rows [q0, q_end) are real
-  const int k_end = min(len_k, q_end);              // keys [0, k_end) are visible to some row
+  const int k_end = min(len_k, off + q_end);        // keys [0, k_end) are visible to some row
   const int nsteps = (k_end + kKeys - 1) / kKeys;
 
   // ---- Q^T of both column groups as B operands: column r of group g is row
@@ -394,11 +420,14 @@ __global__ __launch_bounds__(kWaves * 64, kGroups <= 2 ? 2 : 1) void prefill_att
       reinterpret_cast<const char*>(a.k + ((int64_t)k_base * a.num_kv_heads + kvh) * kPieces);
   const char* v_head =
       reinterpret_cast<const char*>(a.v + ((int64_t)k_base * a.num_kv_heads + kvh) * kPieces);
+  const const_i32_ptr table =
+      PAGED ? (const_i32_ptr)(uintptr_t)(a.block_tables + (int64_t)seq * a.max_blocks) : cu_q;
 
   const lds_ptr k_lds = (lds_ptr)k_ring;
   const lds_ptr v_lds = (lds_ptr)v_ring;
-  const TileCopier copier = {k_head, v_head, row_bytes, (uint32_t)(uintptr_t)k_lds,
-                             (uint32_t)(uintptr_t)v_lds, k_end - 1, nsteps - 1, wave, lane};
+  const TileCopier<PAGED> copier = {k_head, v_head, row_bytes, (uint32_t)(uintptr_t)k_lds,
+                                    (uint32_t)(uintptr_t)v_lds, k_end - 1, nsteps - 1, wave, lane,
+                                    table, a.block_size, a.num_blocks};
 
   const float sl2 = a.scale_log2e;
   f32x4 acc[kGroups][8], lacc[kGroups];
@@ -435,8 +464,8 @@ __global__ __launch_bounds__(kWaves * 64, kGroups <= 2 ? 2 : 1) void prefill_att
   // masked ones (the diagonal tile, or one that reaches past the last key),
   // then tiles whose keys no row of the wave sees, where it only helps to copy.
   // Separate loops rather than a branch inside one keep the accumulators in place.
-  const int n_active = min(nsteps, (wave_row0 + kRowsPerWave - 1) / kKeys + 1);
-  const int n_plain = min(min(wave_row0, k_end) / kKeys, n_active);
+  const int n_active = min(nsteps, (off + wave_row0 + kRowsPerWave - 1) / kKeys + 1);
+  const int n_plain = min(min(off + wave_row0, k_end) / kKeys, n_active);
 
   int k_stage = 0;   // ring slot of K of tile i
   int v_stage = 0;   // ring slot of V of tile i (tile i-1 sits one slot before)
@@ -473,7 +502,7 @@ __global__ __launch_bounds__(kWaves * 64, kGroups <= 2 ? 2 : 1) void prefill_att
     scores_of_tile<F16>(k_lds + k_stage * kTileBytes, qreg, sc, r, kg);
     accumulate_tile<F16>(NVJ_V_BEFORE(), pb, acc, lacc, r, kg);
     __builtin_amdgcn_s_setprio(0);
-    probabilities_of_tile<true, F16>(sc, pb, acc, lacc, m_run, mneg, sl2, r, kg, wave_row0 - ks,
+    probabilities_of_tile<true, F16>(sc, pb, acc, lacc, m_run, mneg, sl2, r, kg, off + wave_row0 - ks,
                                 k_end - 1 - ks);
     __builtin_amdgcn_s_setprio(1);
     NVJ_NEXT_TILE(i);
@@ -506,6 +535,23 @@ __global__ __launch_bounds__(kWaves * 64, kGroups <= 2 ? 2 : 1) void prefill_att
   }
 }
 
+int launch_prefill(hipStream_t stream, PrefillArgs a, bool paged, int32_t total_q_tokens,
+                   int32_t dtype) {
+  // every sequence adds at most one partly filled tile
+  const int64_t tiles = (int64_t)total_q_tokens / kBM + a.batch;
+  if (tiles > INT32_MAX) return NVJ_ERR_BAD_SHAPE;
+  const int64_t items = tiles * a.num_heads;
+  if (items > INT32_MAX - 8) return NVJ_ERR_BAD_SHAPE;
+  const dim3 grid((unsigned)((items + 7) / 8 * 8)), block(kWaves * 64);
+  const int nt = (int)tiles;
+  const bool f16 = dtype == NVJ_DTYPE_F16;
+  if (paged && f16) prefill_attention_kernel<true, true><<<grid, block, 0, stream>>>(a, nt);
+  else if (paged) prefill_attention_kernel<false, true><<<grid, block, 0, stream>>>(a, nt);
+  else if (f16) prefill_attention_kernel<true, false><<<grid, block, 0, stream>>>(a, nt);
+  else prefill_attention_kernel<false, false><<<grid, block, 0, stream>>>(a, nt);
+  return hipGetLastError() == hipSuccess ? NVJ_OK : NVJ_ERR_LAUNCH;
+}
+
 }  // namespace
 
 extern "C" int nvj_prefill_attention_launch(void* stream, const void* q, const void* k,
@@ -526,7 +572,7 @@ extern "C" int nvj_prefill_attention_launch(void* stream, const void* q, const v
   if ((reinterpret_cast<uintptr_t>(q) | reinterpret_cast<uintptr_t>(k) |
        reinterpret_cast<uintptr_t>(v) | reinterpret_cast<uintptr_t>(out)) & 15u)
     return NVJ_ERR_BAD_SHAPE;
-  PrefillArgs a;
+  PrefillArgs a = {};
   a.q = static_cast<const uint4*>(q);
   a.k = static_cast<const uint4*>(k);
   a.v = static_cast<const uint4*>(v);
@@ -538,16 +584,46 @@ extern "C" int nvj_prefill_attention_launch(void* stream, const void* q, const v
   a.num_kv_heads = num_kv_heads;
   a.group = num_heads / num_kv_heads;
   a.scale_log2e = scale * kLog2e;
-  // every sequence adds at most one partly filled tile
-  const int64_t tiles = (int64_t)total_q_tokens / kBM + batch;
-  if (tiles > INT32_MAX) return NVJ_ERR_BAD_SHAPE;
-  const int64_t items = tiles * num_heads;
-  if (items > INT32_MAX - 8) return NVJ_ERR_BAD_SHAPE;
-  const unsigned grid = (unsigned)((items + 7) / 8 * 8);
-  const auto hs = static_cast<hipStream_t>(stream);
-  if (dtype == NVJ_DTYPE_F16)
-    prefill_attention_kernel<true><<<dim3(grid), dim3(kWaves * 64), 0, hs>>>(a, (int)tiles);
-  else
-    prefill_attention_kernel<false><<<dim3(grid), dim3(kWaves * 64), 0, hs>>>(a, (int)tiles);
-  return hipGetLastError() == hipSuccess ? NVJ_OK : NVJ_ERR_LAUNCH;
+  return launch_prefill(static_cast<hipStream_t>(stream), a, false, total_q_tokens, dtype);
+}
+
+extern "C" int nvj_paged_prefill_attention_launch(
+    void* stream, const void* q, const void* k_cache, const void* v_cache,
+    const int32_t* block_tables, const int32_t* cu_seqlens_q, const int32_t* cu_seqlens_k,
+    void* out, int32_t total_q_tokens, int32_t batch, int32_t num_heads, int32_t num_kv_heads,
+    int32_t head_dim, int32_t block_size, int32_t max_blocks, int32_t num_blocks, float scale,
+    int32_t dtype) {
+  if (dtype != NVJ_DTYPE_BF16 && dtype != NVJ_DTYPE_F16) return NVJ_ERR_BAD_DTYPE;
+  if (total_q_tokens < 0 || batch < 0 || num_heads <= 0 || num_kv_heads <= 0 || block_size <= 0 ||
+      max_blocks < 0 || num_blocks <= 0)
+    return NVJ_ERR_BAD_SHAPE;
+  if (num_heads % num_kv_heads != 0) return NVJ_ERR_BAD_SHAPE;
+  if (head_dim != kD || block_size % kKeys != 0) return NVJ_ERR_UNSUPPORTED;
+  if (num_kv_heads > 32768) return NVJ_ERR_UNSUPPORTED;   // a key row stays below 2^24 bytes
+  if ((int64_t)max_blocks * block_size > INT32_MAX) return NVJ_ERR_BAD_SHAPE;
+  if (!(scale >= 0.f)) return NVJ_ERR_BAD_SHAPE;
+  if (total_q_tokens == 0 || batch == 0) return NVJ_OK;
+  if (!q || !k_cache || !v_cache || !cu_seqlens_q || !cu_seqlens_k || !out)
+    return NVJ_ERR_NULL_POINTER;
+  if (max_blocks > 0 && !block_tables) return NVJ_ERR_NULL_POINTER;
+  if ((reinterpret_cast<uintptr_t>(q) | reinterpret_cast<uintptr_t>(k_cache) |
+       reinterpret_cast<uintptr_t>(v_cache) | reinterpret_cast<uintptr_t>(out)) & 15u)
+    return NVJ_ERR_BAD_SHAPE;
+  PrefillArgs a = {};
+  a.q = static_cast<const uint4*>(q);
+  a.k = static_cast<const uint4*>(k_cache);
+  a.v = static_cast<const uint4*>(v_cache);
+  a.out = static_cast<uint4*>(out);
+  a.cu_q = cu_seqlens_q;
+  a.cu_k = cu_seqlens_k;
+  a.batch = batch;
+  a.num_heads = num_heads;
+  a.num_kv_heads = num_kv_heads;
+  a.group = num_heads / num_kv_heads;
+  a.scale_log2e = scale * kLog2e;
+  a.block_tables = block_tables;
+  a.block_size = block_size;
+  a.max_blocks = max_blocks;
+  a.num_blocks = num_blocks;
+  return launch_prefill(static_cast<hipStream_t>(stream), a, true, total_q_tokens, dtype);
 }

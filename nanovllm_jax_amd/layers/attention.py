@@ -19,7 +19,7 @@ import torch
 from .. import _lib
 from ..utils.context import AttentionContext
 from .paged_attention import paged_attention
-from .prefill_attention import variable_length_attention_prefill
+from .prefill_attention import paged_prefill_attention, variable_length_attention_prefill
 
 __all__ = ["store_kv_to_cache", "Attention"]
 
@@ -113,6 +113,17 @@ class Attention:
         """Variable-length causal attention over the packed prompt rows
         (layers/attention.py:331-364)."""
         dt = self.k_cache.dtype           # the model dtype: bf16 or float16
+        if context.block_tables is not None:
+            # prompt rows behind a cached prefix: the reference's filler sets
+            # block_tables exactly then (engine/model_runner.py:309-312); keys and
+            # values, the rows just stored included, come from the paged cache
+            k_cache, v_cache = self.k_cache, self.v_cache
+            if k_cache.dim() == 3:
+                shape = (-1, self.block_size, self.num_kv_heads, self.head_dim)
+                k_cache, v_cache = k_cache.view(shape), v_cache.view(shape)
+            return paged_prefill_attention(q.to(dt).contiguous(), k_cache, v_cache,
+                                           context.block_tables, context.cu_seqlens_q,
+                                           context.cu_seqlens_k, self.scale)
         return variable_length_attention_prefill(
             q.to(dt).contiguous(), k.to(dt).contiguous(), v.to(dt).contiguous(),
             context.cu_seqlens_q, context.cu_seqlens_k, context.max_seqlen_q,

@@ -558,6 +558,48 @@ def variable_length_attention_prefill_ref(q, k, v, cu_seqlens_q, cu_seqlens_k, s
     return out if return_f32 else encode(out)
 
 
+def paged_prefill_attention_ref(q, k_cache, v_cache, block_tables, cu_seqlens_q, cu_seqlens_k,
+                                scale, return_f32: bool = False, dtype: str = "bf16"):
+    """Prefill attention behind a cached prefix.  The reference prepares this case
+    (``engine/model_runner.py:286-312``: ``seqlen_k = len(seq)``, ``seqlen_q`` without
+    the cached tokens, ``block_tables`` set) but its attention call never reads the
+    cached keys, so there is no reference behaviour to restate beyond the
+    mathematics: the ``len_q`` query rows of a sequence are its last ``len_q``
+    positions, row j attends the keys at positions ``<= len_k - len_q + j``, all
+    ``len_k`` keys and values gathered from the pages (``layers/attention.py:80-122``),
+    and the attention itself as in ``variable_length_attention_prefill_ref``."""
+    decode, encode = _codec(dtype)
+    q = np.asarray(q)
+    T, Hq, D = q.shape
+    NB, bs, Hkv, _ = k_cache.shape
+    G = Hq // Hkv
+    cu_q = np.asarray(cu_seqlens_q, dtype=np.int64)
+    cu_k = np.asarray(cu_seqlens_k, dtype=np.int64)
+    bt = np.asarray(block_tables)
+    out = np.zeros((T, Hq, D), dtype=np.float32)
+    scale = np.float32(scale)
+    for i in range(len(cu_q) - 1):
+        lq = int(cu_q[i + 1] - cu_q[i])
+        lk = min(max(int(cu_k[i + 1] - cu_k[i]), 0), bt.shape[1] * bs)
+        if lq <= 0 or lk <= 0:
+            continue
+        pages = np.clip(bt[i, :-(-lk // bs)], 0, NB - 1)
+        ks = decode(k_cache[pages].reshape(-1, Hkv, D)[:lk])
+        vs = decode(v_cache[pages].reshape(-1, Hkv, D)[:lk])
+        qs = decode(q[cu_q[i]:cu_q[i + 1]]).reshape(lq, Hkv, G, D)
+        off = max(lk - lq, 0)
+        mask = (off + np.arange(lq))[:, None] >= np.arange(lk)[None, :]
+        s = np.einsum("qhgd,khd->hgqk", qs, ks, dtype=np.float32) * scale
+        s = np.where(mask[None, None], s, np.float32(-1e30))
+        s = s - s.max(axis=-1, keepdims=True)
+        e = np.where(mask[None, None], np.exp(s, dtype=np.float32), np.float32(0))
+        p = e / e.sum(axis=-1, keepdims=True, dtype=np.float32)
+        p = decode(encode(p))
+        o = np.einsum("hgqk,khd->qhgd", p, vs, dtype=np.float32)
+        out[cu_q[i]:cu_q[i + 1]] = o.reshape(lq, Hq, D)
+    return out if return_f32 else encode(out)
+
+
 def textbook_prefill_f64(q, k, v, cu_seqlens_q, cu_seqlens_k, scale):
     """Causal softmax(q K^T scale) V per (sequence, head, query row) in float64
     with plain loops: the brute force the restatement above is pinned against."""

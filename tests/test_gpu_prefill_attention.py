@@ -125,3 +125,122 @@ def test_attention_layer_prefill_then_decode():
     dout = attn(dq, bits_to_torch(k[last], dev), bits_to_torch(v[last], dev), dctx)
     torch.cuda.synchronize()
     assert_close_bf16(torch_to_bits(dout), want[last], what="decode == last prefill row")
+
+
+# ---- prefill behind a cached prefix: keys and values from the paged cache ----
+def _paged_problem(seed, lens_k, lens_q, Hq, Hkv, bs, extra_pages=3):
+    from nanovllm_jax_amd.workloads import draw_bf16_bits
+    rng = np.random.Generator(np.random.PCG64(seed))
+    D = 128
+    B = len(lens_k)
+    nblk = [-(-n // bs) for n in lens_k]
+    NB = sum(nblk) + extra_pages
+    kc, vc = draw_bf16_bits(rng, (NB, bs, Hkv, D)), draw_bf16_bits(rng, (NB, bs, Hkv, D))
+    cu_q = np.concatenate([[0], np.cumsum(lens_q)]).astype(np.int32)
+    cu_k = np.concatenate([[0], np.cumsum(lens_k)]).astype(np.int32)
+    q = draw_bf16_bits(rng, (max(int(cu_q[-1]), 1), Hq, D), 2.0)[:int(cu_q[-1])]
+    bt = np.full((B, max(max(nblk), 1) + 1), -1, np.int32)       # one padding column
+    pages = rng.permutation(NB)
+    used = 0
+    for i, n in enumerate(nblk):
+        bt[i, :n] = pages[used:used + n]
+        used += n
+    return q, kc, vc, bt, cu_q, cu_k
+
+
+def run_hip_paged(q, kc, vc, bt, cu_q, cu_k, scale):
+    import torch
+    from nanovllm_jax_amd import paged_prefill_attention
+    dev = "cuda:0"
+    out = paged_prefill_attention(bits_to_torch(q, dev), bits_to_torch(kc, dev),
+                                  bits_to_torch(vc, dev), torch.from_numpy(bt).to(dev),
+                                  torch.from_numpy(cu_q).to(dev), torch.from_numpy(cu_k).to(dev),
+                                  scale)
+    torch.cuda.synchronize()
+    return torch_to_bits(out)
+
+
+@pytest.mark.parametrize("Hq,Hkv,bs", [(8, 2, 32), (16, 8, 64), (32, 8, 256), (4, 4, 96)])
+def test_paged_prefill_behind_a_cached_prefix(Hq, Hkv, bs):
+    """Prompt chunks of many lengths behind prefixes of many lengths (none, shorter
+    and longer than a page, ending on and off page and tile boundaries), pages in
+    random order, padding table entries, garbage in unused pages."""
+    print(f"case paged prefill Hq={Hq} Hkv={Hkv} bs={bs}", flush=True)
+    from oracle.paged_attention_oracle import paged_prefill_attention_ref
+    lens_q = [1, 33, 128, 129, 40, 300, 5, 64]
+    prefix = [0, 31, 32, 500, 257, 0, 700, 64]
+    lens_k = [a + b for a, b in zip(lens_q, prefix)]
+    q, kc, vc, bt, cu_q, cu_k = _paged_problem(70 + Hq + bs, lens_k, lens_q, Hq, Hkv, bs)
+    scale = 128 ** -0.5
+    want = paged_prefill_attention_ref(q, kc, vc, bt, cu_q, cu_k, scale)
+    got = run_hip_paged(q, kc, vc, bt, cu_q, cu_k, scale)
+    assert_close_bf16(got, want, what="paged prefill")
+    # poison everything no live key sits on: the result must not move
+    live = np.zeros(kc.shape[:2], bool)
+    for i, n in enumerate(lens_k):
+        for p in range(n):
+            live[bt[i, p // bs], p % bs] = True
+    kc2, vc2 = kc.copy(), vc.copy()
+    kc2[~live] = 0x7FC0
+    vc2[~live] = 0x7FC0                                           # NaN
+    bt2 = np.where(bt < 0, 10 ** 6, bt).astype(np.int32)          # padding entries out of range
+    got2 = run_hip_paged(q, kc2, vc2, bt2, cu_q, cu_k, scale)
+    assert np.array_equal(got, got2), "something outside the live keys was read"
+
+
+def test_paged_prefill_without_prefix_equals_packed_prefill_bit_for_bit():
+    print("case paged prefill == packed prefill", flush=True)
+    lens = [300, 77, 1, 129]
+    Hq, Hkv, bs = 16, 8, 64
+    q, kc, vc, bt, cu_q, cu_k = _paged_problem(81, lens, lens, Hq, Hkv, bs)
+    # the packed rows are the live cache rows in sequence order
+    k = np.concatenate([kc[bt[i, p // bs], p % bs][None] for i, n in enumerate(lens) for p in range(n)])
+    v = np.concatenate([vc[bt[i, p // bs], p % bs][None] for i, n in enumerate(lens) for p in range(n)])
+    scale = 0.11
+    packed = run_hip(q, k, v, cu_q, cu_k, scale)
+    paged = run_hip_paged(q, kc, vc, bt, cu_q, cu_k, scale)
+    assert np.array_equal(packed, paged)
+
+
+def test_attention_layer_prefill_with_cached_prefix():
+    """Attention.__call__ with a prefill context that carries block_tables (the
+    reference's filler sets them when a prefix is cached): the chunk's K/V rows are
+    stored, then the chunk attends over prefix + chunk from the cache; a decode step
+    with the chunk's last token as the query sees the same keys."""
+    print("case Attention prefill behind a cached prefix", flush=True)
+    import torch
+    from nanovllm_jax_amd import Attention, create_decode_context, create_prefill_context
+    from nanovllm_jax_amd.workloads import draw_bf16_bits
+    from oracle.paged_attention_oracle import (paged_prefill_attention_ref,
+                                               store_kv_to_cache_ref)
+    Hq, Hkv, D, bs = 16, 8, 128, 64
+    prefix, chunk = [100, 0, 64], [60, 130, 7]
+    lens_k = [a + b for a, b in zip(prefix, chunk)]
+    q, kc, vc, bt, cu_q, cu_k = _paged_problem(82, lens_k, chunk, Hq, Hkv, bs)
+    rng = np.random.Generator(np.random.PCG64(83))
+    k_new = draw_bf16_bits(rng, (int(cu_q[-1]), Hkv, D))
+    v_new = draw_bf16_bits(rng, (int(cu_q[-1]), Hkv, D))
+    slots = np.concatenate([bt[i, np.arange(prefix[i], lens_k[i]) // bs] * bs +
+                            np.arange(prefix[i], lens_k[i]) % bs for i in range(3)]).astype(np.int32)
+    dev = "cuda:0"
+    up = lambda a: torch.from_numpy(a).to(dev)
+    attn = Attention(Hq, D, D ** -0.5, Hkv, bs)
+    attn.set_kv_cache(bits_to_torch(kc, dev), bits_to_torch(vc, dev))
+    ctx = create_prefill_context(up(cu_q), up(cu_k), max(chunk), max(lens_k), up(slots),
+                                 block_tables=up(bt))
+    out = attn(bits_to_torch(q, dev), bits_to_torch(k_new, dev), bits_to_torch(v_new, dev), ctx)
+    torch.cuda.synchronize()
+    flat = (-1, Hkv, D)
+    wk, wv = store_kv_to_cache_ref(k_new, v_new, kc.reshape(flat), vc.reshape(flat), slots,
+                                   negative_slots="skip")
+    assert np.array_equal(torch_to_bits(attn.k_cache).reshape(flat), wk)
+    want = paged_prefill_attention_ref(q, wk.reshape(kc.shape), wv.reshape(vc.shape), bt, cu_q,
+                                       cu_k, D ** -0.5)
+    assert_close_bf16(torch_to_bits(out), want, what="layer prefill behind a prefix")
+    last = cu_q[1:] - 1
+    dctx = create_decode_context(up(np.array(lens_k, np.int32)), up(np.full(3, -1, np.int32)),
+                                 up(bt))
+    dout = attn(bits_to_torch(q[last], dev), bits_to_torch(k_new[last], dev),
+                bits_to_torch(v_new[last], dev), dctx)
+    torch.cuda.synchronize()
+    assert_close_bf16(torch_to_bits(dout), want[last], what="decode == last chunk row")

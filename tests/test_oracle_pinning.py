@@ -498,3 +498,51 @@ def test_c_oracle_float16_matches_the_numpy_restatement():
     assert np.allclose(got, want, rtol=1e-5, atol=1e-6)
     got_bits = c_oracle.paged_decode(q, kc, vc, bt, ctx, 0.09, bs, dtype="f16")
     assert np.array_equal(got_bits, f32_to_f16_bits(got))
+
+
+def test_paged_prefill_oracle_against_float64_and_the_packed_one():
+    """The cached-prefix prefill restatement: equal to the packed one when nothing
+    is cached, and to a float64 brute force (bottom-right aligned causal mask over
+    the gathered pages) when a prefix is."""
+    from oracle.paged_attention_oracle import (paged_prefill_attention_ref,
+                                               variable_length_attention_prefill_ref)
+    from nanovllm_jax_amd.workloads import draw_bf16_bits
+    rng = np.random.Generator(np.random.PCG64(91))
+    Hq, Hkv, D, bs, NB = 4, 2, 128, 32, 12
+    lens_k, lens_q = [70, 33, 5], [20, 33, 1]
+    cu_q = np.concatenate([[0], np.cumsum(lens_q)]).astype(np.int32)
+    cu_k = np.concatenate([[0], np.cumsum(lens_k)]).astype(np.int32)
+    kc, vc = draw_bf16_bits(rng, (NB, bs, Hkv, D)), draw_bf16_bits(rng, (NB, bs, Hkv, D))
+    q = draw_bf16_bits(rng, (int(cu_q[-1]), Hq, D), 2.0)
+    bt = np.full((3, 3), -1, np.int32)
+    pages = rng.permutation(NB)
+    used = 0
+    for i, n in enumerate(lens_k):
+        nb = -(-n // bs)
+        bt[i, :nb] = pages[used:used + nb]
+        used += nb
+    got = paged_prefill_attention_ref(q, kc, vc, bt, cu_q, cu_k, 0.1, return_f32=True)
+    qf = bf16_bits_to_f32(q).astype(np.float64)
+    for i in range(3):
+        lk, lq = lens_k[i], lens_q[i]
+        kk = bf16_bits_to_f32(kc[bt[i, :-(-lk // bs)]].reshape(-1, Hkv, D)[:lk]).astype(np.float64)
+        vv = bf16_bits_to_f32(vc[bt[i, :-(-lk // bs)]].reshape(-1, Hkv, D)[:lk]).astype(np.float64)
+        for j in range(lq):
+            n = lk - lq + j + 1
+            for h in range(Hq):
+                lg = 0.1 * (kk[:n, h // 2] @ qf[cu_q[i] + j, h])
+                w = np.exp(lg - lg.max()); w /= w.sum()
+                assert np.allclose(got[cu_q[i] + j, h], w @ vv[:n, h // 2], atol=1e-2), (i, j, h)
+    # nothing cached: the packed restatement on the same rows
+    lens = [40, 7]
+    cu = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
+    k = draw_bf16_bits(rng, (47, Hkv, D)); v = draw_bf16_bits(rng, (47, Hkv, D))
+    q = draw_bf16_bits(rng, (47, Hq, D))
+    kc2 = np.zeros((4, bs, Hkv, D), np.uint16); vc2 = np.zeros_like(kc2)
+    bt2 = np.array([[2, 0], [3, -1]], np.int32)
+    for i, n in enumerate(lens):
+        for p in range(n):
+            kc2[bt2[i, p // bs], p % bs] = k[cu[i] + p]; vc2[bt2[i, p // bs], p % bs] = v[cu[i] + p]
+    a = paged_prefill_attention_ref(q, kc2, vc2, bt2, cu, cu, 0.1)
+    b = variable_length_attention_prefill_ref(q, k, v, cu, cu, 0.1)
+    assert np.array_equal(a, b)
