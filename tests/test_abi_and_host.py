@@ -66,6 +66,12 @@ def test_argument_validation_without_a_gpu():
     assert P(None, x, x, x, x, x, x, x, 1 << 30, 2, 32, 8, 128, 256, 4, 16, 0.1, 0, 2, valu) == -3
     assert P(None, x, x, x, x, x, x, x, 1 << 30, 2, 32, 8, 128, 256, 4, 16, 0.1, 256, 0, valu) == -3
     assert P(None, x, x, x, x, x, x, x, 1 << 30, 0, 32, 8, 128, 256, 4, 16, 0.1, 0, 0, valu) == 0
+    PP = lib.nvj_paged_prefill_attention_launch
+    assert PP(None, x, x, x, x, x, x, x, 10, 2, 32, 8, 128, 48, 4, 16, 0.1, 0) == -3   # page % 32
+    assert PP(None, x, x, x, x, x, x, x, 10, 2, 32, 8, 64, 64, 4, 16, 0.1, 0) == -3    # head_dim
+    assert PP(None, x, x, x, x, x, x, x, 10, 2, 32, 8, 128, 64, 4, 16, 0.1, 1) == -6   # f32
+    assert PP(None, x, x, x, 0, x, x, x, 10, 2, 32, 8, 128, 64, 4, 16, 0.1, 0) == -1   # no tables
+    assert PP(None, x, x, x, x, x, x, x, 0, 2, 32, 8, 128, 64, 4, 16, 0.1, 0) == 0     # no rows
     S = lib.nvj_store_kvcache_launch
     assert S(None, 0, 0, 0, 0, 0, 0, 8, 128, 1024, 0, 0, 0) == 0       # no tokens
     assert S(None, 0x1000, 0x1000, 0x1000, 0x1000, 0x1000, 4, 8, 128, 1024, 7, 0, 0) == -6
