@@ -32,7 +32,8 @@ from ..layers.attention import Attention
 from ..layers.layernorm import rms_norm
 from ..layers.paged_attention import (choose_split, paged_attention,
                                       paged_decode_workspace_bytes)
-from ..layers.prefill_attention import variable_length_attention_prefill
+from ..layers.prefill_attention import (paged_prefill_attention,
+                                        variable_length_attention_prefill)
 from ..layers.qk_rope_store import qk_norm_rope_store
 from ..utils.context import AttentionContext, create_decode_context, create_prefill_context
 
@@ -83,26 +84,34 @@ def prepare_decode(last_tokens, seq_lens, block_tables, block_size):
     return input_ids, positions, context_lens, slot_mapping, prepare_block_tables(block_tables)
 
 
-def prepare_prefill(token_lists, block_tables, block_size):
-    """Host filler of one prefill step without prefix caching
-    (``engine/model_runner.py:248-332`` with ``num_cached_tokens == 0``): packed
-    ``input_ids`` and ``positions = 0 .. len-1``, ``cu_seqlens_q == cu_seqlens_k``,
-    and per sequence the slots of its pages in order, ``block_size`` per page
-    except ``last_block_num_tokens`` in the last (:300-309)."""
+def prepare_prefill(token_lists, block_tables, block_size, num_cached_tokens=None):
+    """Host filler of one prefill step (``engine/model_runner.py:248-332``): packed
+    ``input_ids`` and ``positions`` of the tokens that are not cached yet,
+    ``cu_seqlens_q`` over those, ``cu_seqlens_k`` over whole sequences, and per
+    sequence the slots of the new tokens, page by page (:300-309).
+    ``num_cached_tokens[i]`` leading tokens of sequence i already sit in the cache
+    (0 everywhere by default); unlike the reference's block-granular prefix cache
+    it may be any count.  Returns ``(input_ids, positions, cu_seqlens_q,
+    cu_seqlens_k, slot_mapping, max_seqlen_q, max_seqlen_k)``."""
     lens = [len(t) for t in token_lists]
-    cu = np.zeros(len(lens) + 1, np.int32)
-    cu[1:] = np.cumsum(lens)
-    input_ids = np.concatenate([np.asarray(t, np.int32) for t in token_lists])
-    positions = np.concatenate([np.arange(n, dtype=np.int32) for n in lens])
+    cached = list(num_cached_tokens) if num_cached_tokens is not None else [0] * len(lens)
+    new = [n - c for n, c in zip(lens, cached)]
+    cu_q = np.zeros(len(lens) + 1, np.int32)
+    cu_q[1:] = np.cumsum(new)
+    cu_k = np.zeros(len(lens) + 1, np.int32)
+    cu_k[1:] = np.cumsum(lens)
+    input_ids = (np.concatenate([np.asarray(t[c:], np.int32) for t, c in zip(token_lists, cached)])
+                 if lens else np.zeros(0, np.int32))
+    positions = (np.concatenate([np.arange(c, n, dtype=np.int32) for n, c in zip(lens, cached)])
+                 if lens else np.zeros(0, np.int32))
     slots = []
-    for n, table in zip(lens, block_tables):
-        num_blocks = -(-n // block_size)
-        for i in range(num_blocks):
-            start = table[i] * block_size
-            block_len = block_size if i != num_blocks - 1 else n - (num_blocks - 1) * block_size
-            slots.append(np.arange(start, start + block_len, dtype=np.int32))
+    for n, c, table in zip(lens, cached, block_tables):
+        pos = np.arange(c, n)
+        slots.append((np.asarray(table, np.int64)[pos // block_size] * block_size +
+                      pos % block_size).astype(np.int32))
     slot_mapping = np.concatenate(slots) if slots else np.zeros(0, np.int32)
-    return input_ids, positions, cu, slot_mapping, max(lens) if lens else 0
+    return (input_ids, positions, cu_q, cu_k, slot_mapping, max(new) if new else 0,
+            max(lens) if lens else 0)
 
 
 def advance_decode(next_tokens, input_ids, positions, context: AttentionContext, block_size):
@@ -245,7 +254,13 @@ class DecodeStepRunner:
                                        c.rms_norm_eps, attn.k_cache, attn.v_cache,
                                        context.slot_mapping, c.num_heads, c.num_kv_heads,
                                        c.head_dim)
-                if context.is_prefill:
+                if context.is_prefill and context.block_tables is not None:
+                    # prompt rows behind a cached prefix: keys and values, the rows the
+                    # fused launch just stored included, come from the paged cache
+                    o = paged_prefill_attention(q, attn.k_cache, attn.v_cache,
+                                                context.block_tables, context.cu_seqlens_q,
+                                                context.cu_seqlens_k, attn.scale)
+                elif context.is_prefill:
                     # K/V of the prompt rows were normalised, rotated and stored by
                     # the fused launch; the prefill kernel wants them packed, so
                     # they are gathered back from the cache rows just written
@@ -289,13 +304,18 @@ class DecodeStepRunner:
         split = choose_split(ctx, self.cfg.num_kv_heads, self.cfg.num_heads)
         return t(ids), t(pos), create_decode_context(t(ctx), t(slots), t(bt), split)
 
-    def make_prefill_inputs(self, token_lists, block_tables):
-        ids, pos, cu, slots, max_len = prepare_prefill(token_lists, block_tables,
-                                                       self.cfg.block_size)
+    def make_prefill_inputs(self, token_lists, block_tables, num_cached_tokens=None):
+        """Prefill inputs; with ``num_cached_tokens`` the context carries the block
+        tables (as the reference's does when a prefix is cached,
+        ``engine/model_runner.py:309-312``) and attention reads keys and values
+        from the paged cache."""
+        ids, pos, cu_q, cu_k, slots, max_q, max_k = prepare_prefill(
+            token_lists, block_tables, self.cfg.block_size, num_cached_tokens)
         d = self.device
         t = lambda a: torch.from_numpy(a).to(d)
-        cu_t = t(cu)
-        return t(ids), t(pos), create_prefill_context(cu_t, cu_t, max_len, max_len, t(slots))
+        bt = t(prepare_block_tables(block_tables)) if num_cached_tokens is not None else None
+        return t(ids), t(pos), create_prefill_context(t(cu_q), t(cu_k), max_q, max_k, t(slots),
+                                                      block_tables=bt)
 
     def step(self, input_ids, positions, context):
         """Eager decode step: logits -> greedy token ids [batch] int64."""

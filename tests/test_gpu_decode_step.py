@@ -225,3 +225,42 @@ def test_prefill_then_decode_equals_one_longer_prefill(fused):
         scale = want.abs().max().item()
         print(f"  step {step}: max |logit diff| {err:.3e} (max |logit| {scale:.2f})", flush=True)
         assert err <= 0.015 * scale + 0.01
+
+
+@pytest.mark.parametrize("fused", [True, False])
+def test_prefill_in_two_chunks_equals_one_prefill(fused):
+    """Chunked prefill over the whole layer stack: the first part of every prompt
+    is prefilled and cached, the rest is prefilled behind it (keys and values of
+    both parts read from the paged cache, positions and slots of the second part
+    only), and the logits of the last tokens match a one-shot prefill."""
+    print(f"case prefill in two chunks fused={fused}", flush=True)
+    cfg, runner = _small_runner(fused)
+    _, check = _small_runner(fused)
+    rng = np.random.Generator(np.random.PCG64(13))
+    lens = [70, 300, 131, 9]
+    first = [64, 129, 0, 8]               # cached before the second chunk (0: nothing)
+    prompts = [rng.integers(0, cfg.vocab_size, n).tolist() for n in lens]
+    pages = rng.permutation(cfg.num_kvcache_blocks).tolist()
+    tables, off = [], 0
+    for n in lens:
+        k = -(-n // cfg.block_size)
+        tables.append(pages[off:off + k]); off += k
+    ids, pos, ctx = check.make_prefill_inputs(prompts, tables)
+    want = check.forward(ids, pos, ctx).float()
+    # chunk 1: the sequences that have a first part
+    part = [i for i, c in enumerate(first) if c > 0]
+    ids, pos, ctx = runner.make_prefill_inputs([prompts[i][:first[i]] for i in part],
+                                               [tables[i] for i in part])
+    runner.forward(ids, pos, ctx)
+    # chunk 2: everything that is left, behind the cached part
+    ids, pos, ctx = runner.make_prefill_inputs(prompts, tables, num_cached_tokens=first)
+    assert ctx.block_tables is not None and int(ctx.cu_seqlens_q[-1]) == sum(lens) - sum(first)
+    got = runner.forward(ids, pos, ctx).float()
+    torch.cuda.synchronize()
+    err = (got - want).abs().max().item()
+    scale = want.abs().max().item()
+    print(f"  max |logit diff| {err:.3e} (max |logit| {scale:.2f})", flush=True)
+    assert err <= 0.015 * scale + 0.01
+    assert torch.equal(got.argmax(-1), want.argmax(-1))
+    # the caches of both runners hold the same rows
+    assert torch.equal(runner.kv_cache, check.kv_cache)
