@@ -102,3 +102,49 @@ def test_prefill_random_case(seed):
     exact = np.asarray(textbook_prefill_f64(q, k, v, cu_q, cu_k, c["scale"]), np.float64)
     err = np.abs(bf16_bits_to_f32(got).astype(np.float64) - exact)
     assert np.all(err <= 1e-2 + 1e-2 * np.abs(exact)), f"seed={seed}: max err {err.max():.3e} vs float64"
+
+
+def _paged_prefill_case(rng):
+    Hkv = int(rng.choice([1, 2, 4, 8]))
+    G = int(rng.choice([1, 2, 4, 8]))
+    bs = int(rng.choice([32, 64, 96, 256]))
+    n = int(rng.integers(1, 6))
+    lens_q = [int(x) for x in rng.choice([0, 1, 2, 31, 32, 33, 127, 128, 129, 200, 257], n)]
+    prefix = [int(x) for x in rng.choice([0, 0, 1, 31, 32, 33, 100, 257, 511], n)]
+    if sum(lens_q) == 0:
+        lens_q[0] = 5
+    scale = float(rng.choice([128 ** -0.5, 0.0, 0.25]))
+    return dict(Hq=Hkv * G, Hkv=Hkv, bs=bs, lens_q=lens_q, prefix=prefix, scale=scale)
+
+
+@pytest.mark.parametrize("seed", range(16))
+def test_paged_prefill_random_case(seed):
+    import torch
+    from nanovllm_jax_amd import paged_prefill_attention
+    from nanovllm_jax_amd.workloads import draw_bf16_bits
+    from oracle.paged_attention_oracle import paged_prefill_attention_ref
+    c = _paged_prefill_case(np.random.Generator(np.random.PCG64(61000 + seed)))
+    print(f"case paged prefill sweep seed={seed} {c}", flush=True)
+    rng = np.random.Generator(np.random.PCG64(62000 + seed))
+    bs, Hq, Hkv = c["bs"], c["Hq"], c["Hkv"]
+    lens_k = [a + b for a, b in zip(c["lens_q"], c["prefix"])]
+    nblk = [-(-n // bs) for n in lens_k]
+    NB = sum(nblk) + 2
+    kc, vc = draw_bf16_bits(rng, (NB, bs, Hkv, 128)), draw_bf16_bits(rng, (NB, bs, Hkv, 128))
+    cu_q = np.concatenate([[0], np.cumsum(c["lens_q"])]).astype(np.int32)
+    cu_k = np.concatenate([[0], np.cumsum(lens_k)]).astype(np.int32)
+    q = draw_bf16_bits(rng, (int(cu_q[-1]), Hq, 128), 2.0)
+    bt = np.full((len(lens_k), max(nblk) + 1), -1, np.int32)
+    pages = rng.permutation(NB)
+    used = 0
+    for i, n in enumerate(nblk):
+        bt[i, :n] = pages[used:used + n]
+        used += n
+    dev = "cuda:0"
+    out = paged_prefill_attention(bits_to_torch(q, dev), bits_to_torch(kc, dev),
+                                  bits_to_torch(vc, dev), torch.from_numpy(bt).to(dev),
+                                  torch.from_numpy(cu_q).to(dev), torch.from_numpy(cu_k).to(dev),
+                                  c["scale"])
+    torch.cuda.synchronize()
+    want = paged_prefill_attention_ref(q, kc, vc, bt, cu_q, cu_k, c["scale"])
+    assert_close_bf16(torch_to_bits(out), want, what=f"paged prefill sweep seed={seed}")
