@@ -191,3 +191,41 @@ def test_attention_layer_with_float16_caches_prefill_then_decode():
                                                bs, dtype="f16")
     err = np.abs(f16_bits_to_f32(_bits(out1)).astype(np.float64) - f16_bits_to_f32(want1))
     assert np.all(err <= 1e-2 + 1e-2 * np.abs(f16_bits_to_f32(want1))), f"decode {err.max():.3e}"
+
+
+def test_paged_prefill_float16():
+    print("case f16 paged prefill", flush=True)
+    import torch
+    from nanovllm_jax_amd import paged_prefill_attention
+    from nanovllm_jax_amd.workloads import draw_bf16_bits
+    from oracle.paged_attention_oracle import (bf16_bits_to_f32, f16_bits_to_f32, f32_to_f16_bits,
+                                               paged_prefill_attention_ref)
+    rng = np.random.Generator(np.random.PCG64(850))
+    Hq, Hkv, D, bs = 8, 2, 128, 64
+    lens_q, prefix = [40, 129, 1], [100, 0, 63]
+    lens_k = [a + b for a, b in zip(lens_q, prefix)]
+    nblk = [-(-n // bs) for n in lens_k]
+    NB = sum(nblk) + 1
+    cv = lambda b: f32_to_f16_bits(bf16_bits_to_f32(b) * np.float32(1.001))
+    kc, vc = cv(draw_bf16_bits(rng, (NB, bs, Hkv, D))), cv(draw_bf16_bits(rng, (NB, bs, Hkv, D)))
+    cu_q = np.concatenate([[0], np.cumsum(lens_q)]).astype(np.int32)
+    cu_k = np.concatenate([[0], np.cumsum(lens_k)]).astype(np.int32)
+    q = cv(draw_bf16_bits(rng, (int(cu_q[-1]), Hq, D), 2.0))
+    bt = np.full((3, max(nblk)), -1, np.int32)
+    pages = rng.permutation(NB)
+    used = 0
+    for i, n in enumerate(nblk):
+        bt[i, :n] = pages[used:used + n]
+        used += n
+    dev = "cuda:0"
+    scale = D ** -0.5
+    out = paged_prefill_attention(_to_f16(q, dev), _to_f16(kc, dev), _to_f16(vc, dev),
+                                  torch.from_numpy(bt).to(dev), torch.from_numpy(cu_q).to(dev),
+                                  torch.from_numpy(cu_k).to(dev), scale)
+    torch.cuda.synchronize()
+    assert out.dtype == torch.float16
+    got = f16_bits_to_f32(_bits(out)).astype(np.float64)
+    want = f16_bits_to_f32(paged_prefill_attention_ref(q, kc, vc, bt, cu_q, cu_k, scale,
+                                                       dtype="f16")).astype(np.float64)
+    err = np.abs(got - want)
+    assert np.all(err <= 1e-2 + 1e-2 * np.abs(want)), f"max err {err.max():.3e}"
