@@ -20,7 +20,7 @@
 extern "C" {
 #endif
 
-#define NVJ_ABI_VERSION 1
+#define NVJ_ABI_VERSION 2
 
 /* exported from the shared library (which is built with hidden visibility) */
 #define NVJ_API __attribute__((visibility("default")))
@@ -33,6 +33,8 @@ extern "C" {
 #define NVJ_ERR_WORKSPACE     -4   /* workspace too small or misaligned             */
 #define NVJ_ERR_LAUNCH        -5   /* hipGetLastError() != hipSuccess after launch  */
 #define NVJ_ERR_BAD_DTYPE     -6   /* unknown element type code                     */
+#define NVJ_ERR_SCRATCH_LIMIT -7   /* nvj_paged_decode_static_launch: the problem needs
+                                      more than NVJ_STATIC_SCRATCH_BYTES of scratch  */
 
 #define NVJ_CHUNK_WHOLE_SEQUENCE (-1)   /* see the split modes of the paged decode */
 
@@ -198,6 +200,36 @@ NVJ_API int nvj_paged_decode_launch_phases(void* stream,
                             int32_t head_dim, int32_t block_size, int32_t max_blocks,
                             int32_t num_blocks, float scale, int32_t chunk, int32_t dtype,
                             uint32_t phases);
+
+/*
+ * nvj_paged_decode_launch with chunk == 0 (balanced split) for callers that
+ * cannot allocate device memory: code running under HIP graph capture, tight
+ * serving loops, harnesses that forbid hipMalloc.  It has no counterpart in the
+ * reference (whose arrays are all allocated by XLA); results are those of
+ * nvj_paged_decode_launch(chunk = 0) bit for bit.
+ *
+ * The split-K partials live in a device array of NVJ_STATIC_SCRATCH_BYTES that is
+ * part of the library image: every GPU the library runs on holds its own copy
+ * from the first call on that GPU until the process ends.  The call itself
+ * allocates and frees nothing (no hipMalloc / hipFree, no allocating library
+ * routine); the first call on a device looks the array's address up once.  The
+ * device that `stream` belongs to must be the current device.
+ *
+ * A problem whose workspace (nvj_paged_decode_workspace_bytes(..., chunk 0))
+ * exceeds NVJ_STATIC_SCRATCH_BYTES is rejected with NVJ_ERR_SCRATCH_LIMIT;
+ * batch 256 with 32 query heads of 128 dims needs 8.5 MB.  All calls on one GPU
+ * share the one array: calls that may overlap in time on the same GPU (two
+ * streams, two threads) race on it and must be serialised by the caller; calls
+ * on one stream are ordered and safe.  Nothing in the array has to survive from
+ * one call to the next.
+ */
+#define NVJ_STATIC_SCRATCH_BYTES (16u << 20)
+NVJ_API int nvj_paged_decode_static_launch(void* stream,
+                            const void* q, const void* k_cache, const void* v_cache,
+                            const int32_t* block_tables, const int32_t* context_lens,
+                            void* out, int32_t batch, int32_t num_heads, int32_t num_kv_heads,
+                            int32_t head_dim, int32_t block_size, int32_t max_blocks,
+                            int32_t num_blocks, float scale, int32_t dtype);
 
 /*
  * Fused per-head QK-RMSNorm + rotary embedding + KV-cache store: everything the

@@ -13,7 +13,7 @@ import threading
 _LIB_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), "_native",
                          "libnvj_paged_attn.so")
 
-NVJ_ABI_VERSION = 1
+NVJ_ABI_VERSION = 2
 NVJ_DTYPE_BF16 = 0
 NVJ_DTYPE_F32 = 1
 NVJ_DTYPE_F16 = 2
@@ -39,6 +39,11 @@ SYMBOLS = {
         _c.c_void_p, _c.c_void_p, _c.c_size_t,
         _c.c_int32, _c.c_int32, _c.c_int32, _c.c_int32, _c.c_int32, _c.c_int32,
         _c.c_int32, _c.c_float, _c.c_int32, _c.c_int32, _c.c_uint32]),
+    "nvj_paged_decode_static_launch": (_c.c_int, [
+        _c.c_void_p, _c.c_void_p, _c.c_void_p, _c.c_void_p, _c.c_void_p, _c.c_void_p,
+        _c.c_void_p,
+        _c.c_int32, _c.c_int32, _c.c_int32, _c.c_int32, _c.c_int32, _c.c_int32,
+        _c.c_int32, _c.c_float, _c.c_int32]),
     "nvj_qk_norm_rope_store_launch": (_c.c_int, [
         _c.c_void_p, _c.c_void_p, _c.c_int64, _c.c_void_p, _c.c_void_p, _c.c_int32, _c.c_void_p,
         _c.c_void_p, _c.c_float, _c.c_void_p, _c.c_void_p, _c.c_void_p, _c.c_void_p,
@@ -58,6 +63,8 @@ SYMBOLS = {
         _c.c_void_p, _c.c_void_p, _c.c_int64, _c.c_void_p, _c.c_int32, _c.c_int32]),
 }
 NVJ_CHUNK_WHOLE_SEQUENCE = -1
+NVJ_STATIC_SCRATCH_BYTES = 16 << 20
+NVJ_ERR_SCRATCH_LIMIT = -7
 NVJ_PHASE_SPLITK = 1
 NVJ_PHASE_COMBINE = 2
 NVJ_PHASE_VALU_PRODUCTS = 4

@@ -35,6 +35,8 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <atomic>
+
 #include "nvj_paged_attn.h"
 
 namespace {
@@ -1285,6 +1287,58 @@ extern "C" int nvj_paged_decode_launch(void* stream, const void* q, const void* 
                                         NVJ_PHASE_SPLITK | NVJ_PHASE_COMBINE);
 }
 
+// ---------------------------------------------------------------------------
+// Entry point that allocates nothing: the balanced split with its workspace in
+// a file-scope device array instead of caller memory.  The array's name is a
+// host-side stand-in; its device address is looked up once per device
+// (hipGetSymbolAddress) and only that address is ever handed to a kernel.
+// ---------------------------------------------------------------------------
+static __device__ __align__(256) unsigned char scratch[NVJ_STATIC_SCRATCH_BYTES];
+
+namespace {
+constexpr int kMaxDevices = 64;
+std::atomic<void*> g_scratch_ptr[kMaxDevices];   // per device: address of its copy of `scratch`
+
+// Device address of the current device's copy of `scratch`.
+int static_scratch_of_current_device(void** out) {
+  int dev = -1;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return NVJ_ERR_LAUNCH;
+  void* p = g_scratch_ptr[dev].load(std::memory_order_acquire);
+  if (p == nullptr) {
+    // every thread that races here gets the same address from the runtime
+    if (hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)) != hipSuccess || p == nullptr)
+      return NVJ_ERR_LAUNCH;
+    g_scratch_ptr[dev].store(p, std::memory_order_release);
+  }
+  *out = p;
+  return NVJ_OK;
+}
+}  // namespace
+
+extern "C" int nvj_paged_decode_static_launch(void* stream, const void* q, const void* k_cache,
+                                              const void* v_cache, const int32_t* block_tables,
+                                              const int32_t* context_lens, void* out,
+                                              int32_t batch, int32_t num_heads,
+                                              int32_t num_kv_heads, int32_t head_dim,
+                                              int32_t block_size, int32_t max_blocks,
+                                              int32_t num_blocks, float scale, int32_t dtype) {
+  void* ws = nullptr;
+  if (batch > 0 && max_blocks > 0) {
+    const size_t need = nvj_paged_decode_workspace_bytes(batch, num_heads, head_dim, max_blocks,
+                                                         block_size, num_kv_heads, 0);
+    // need == 0: invalid arguments, which the launch below reports by name
+    if (need > NVJ_STATIC_SCRATCH_BYTES) return NVJ_ERR_SCRATCH_LIMIT;
+    if (need > 0) {
+      const int rc = static_scratch_of_current_device(&ws);
+      if (rc != NVJ_OK) return rc;
+    }
+  }
+  return nvj_paged_decode_launch(stream, q, k_cache, v_cache, block_tables, context_lens, out, ws,
+                                 ws ? (size_t)NVJ_STATIC_SCRATCH_BYTES : 0, batch, num_heads,
+                                 num_kv_heads, head_dim, block_size, max_blocks, num_blocks, scale,
+                                 0, dtype);
+}
+
 extern "C" const char* nvj_error_string(int code) {
   switch (code) {
     case NVJ_OK: return "ok";
@@ -1294,6 +1348,8 @@ extern "C" const char* nvj_error_string(int code) {
     case NVJ_ERR_WORKSPACE: return "workspace missing, too small or misaligned";
     case NVJ_ERR_LAUNCH: return "kernel launch failed";
     case NVJ_ERR_BAD_DTYPE: return "unknown element type code";
+    case NVJ_ERR_SCRATCH_LIMIT:
+      return "problem needs more than the library's static scratch (NVJ_STATIC_SCRATCH_BYTES)";
     default: return "unknown error code";
   }
 }
