@@ -85,6 +85,24 @@ def timed(fn, steps, torch):
     return start.elapsed_time(end) / steps, (t1 - t0) * 1e3 / steps
 
 
+def timed_in_graph(fn, torch, calls=20, replays=20):
+    """Mean ms per call when `calls` back-to-back calls are replayed from one HIP
+    graph (launch cost of the host binding excluded)."""
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        fn()
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        for _ in range(calls):
+            fn()
+    graph.replay()
+    ms, _ = timed(graph.replay, replays, torch)
+    return ms / calls
+
+
 def cpu_baseline(w, q, kc, vc, budget_s=20.0, dtype="bf16"):
     """The CPU oracle on the host cores (C restatement, OpenMP over
     (sequence, kv head)), same inputs, on a bounded sample: whole calls over
@@ -270,8 +288,7 @@ def main():
               file=sys.stderr)
         return 1
     from nanovllm_jax_amd import _lib, paged_attention, store_kv_to_cache
-    from nanovllm_jax_amd.layers.paged_attention import (choose_split,
-                                                         paged_decode_workspace_bytes)
+    from nanovllm_jax_amd.layers.paged_attention import DecodeWorkspace, choose_split
     from nanovllm_jax_amd.workloads import algorithmic_bytes, make_workload
 
     dev = torch.device("cuda:0")
@@ -290,9 +307,8 @@ def main():
                                                                         f"fixed chunk {chunk}")
     kernel_name = {0: "paged_decode_balanced_kernel", -1: "paged_decode_whole_kernel"}.get(
         chunk, "paged_decode_splitk_kernel")
-    ws = torch.empty(paged_decode_workspace_bytes(w.batch, w.num_heads, w.head_dim, w.max_blocks,
-                                                  w.block_size, w.num_kv_heads, chunk),
-                     dtype=torch.uint8, device=dev)
+    ws = DecodeWorkspace.for_shape(w.batch, w.num_heads, w.head_dim, w.max_blocks, w.block_size,
+                                   w.num_kv_heads, dev, chunk)
     out = torch.empty_like(q)
     kflat = kc.view(-1, w.num_kv_heads, w.head_dim)
     vflat = vc.view(-1, w.num_kv_heads, w.head_dim)
@@ -321,6 +337,7 @@ def main():
     ms_splitk, _ = timed(lambda: decode(_lib.NVJ_PHASE_SPLITK), args.steps, torch)
     ms_combine, _ = timed(lambda: decode(_lib.NVJ_PHASE_COMBINE), args.steps, torch)
     ms_store, _ = timed(store, args.steps, torch)
+    ms_graph = timed_in_graph(decode, torch)
 
     byts = algorithmic_bytes(w.context_lens, w.batch, w.num_heads, w.num_kv_heads, w.head_dim,
                              w.max_blocks)
@@ -333,6 +350,7 @@ def main():
         "warmup": args.warmup, "ms_per_step": round(ms_wall, 5), "higher_is_better": True,
         "scaling": "weak", "vs_baseline": None, "dtype": args.dtype, "data": "synthetic",
         "us_per_call": round(ms_call * 1e3, 2),
+        "us_per_call_in_graph": round(ms_graph * 1e3, 2),
         "pct_of_hbm_peak": round(100.0 * gbps / HBM_PEAK_GBPS, 2),
         "config": {"workload": f"{w.name}: B={w.batch} Hq={w.num_heads} Hkv={w.num_kv_heads} "
                                f"D={w.head_dim} page={w.block_size} "

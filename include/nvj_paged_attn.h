@@ -30,11 +30,13 @@ extern "C" {
 #define NVJ_ERR_NULL_POINTER  -1   /* a required pointer is NULL                    */
 #define NVJ_ERR_BAD_SHAPE     -2   /* negative size, Hq % Hkv != 0, ...             */
 #define NVJ_ERR_UNSUPPORTED   -3   /* head_dim / group size / block size not built  */
-#define NVJ_ERR_WORKSPACE     -4   /* workspace too small or misaligned             */
+#define NVJ_ERR_WORKSPACE     -4   /* workspace missing or too small                */
 #define NVJ_ERR_LAUNCH        -5   /* hipGetLastError() != hipSuccess after launch  */
 #define NVJ_ERR_BAD_DTYPE     -6   /* unknown element type code                     */
 #define NVJ_ERR_SCRATCH_LIMIT -7   /* nvj_paged_decode_static_launch: the problem needs
                                       more than NVJ_STATIC_SCRATCH_BYTES of scratch  */
+#define NVJ_ERR_ALIGNMENT     -8   /* a data pointer is not 16-byte aligned (every
+                                      entry point; int32 metadata needs 4 bytes)    */
 
 #define NVJ_CHUNK_WHOLE_SEQUENCE (-1)   /* see the split modes of the paged decode */
 
@@ -81,12 +83,15 @@ NVJ_API int nvj_store_kvcache_launch(void* stream,
 /*
  * How the positions of a call are split over workgroups is chosen by `chunk`:
  *
- *   chunk == 0  balanced split (the default): the 32-position steps of all
- *               sequences, end to end in batch order, are cut into equal runs,
- *               one per workgroup and at most one workgroup per CU (256), at
- *               least 128 positions each.  The kernel derives the cut from
- *               context_lens on the device, so ragged batches are balanced
- *               without the host knowing the lengths.
+ *   chunk == 0  balanced split (the default), ONE launch for any mix of
+ *               lengths: the 32-position steps of all (sequence, head group)
+ *               rows, end to end, are cut into equal runs, one per wave, at
+ *               most one 8-wave workgroup per CU.  The kernel derives the cut
+ *               from context_lens on the device, so ragged batches are
+ *               balanced without the host knowing the lengths; a row that
+ *               fits one workgroup is finished there, a row shared by several
+ *               is merged by the wave that completes it (counters in the
+ *               workspace), without a second launch.
  *   chunk  > 0  fixed split: workgroup (b, c) takes positions
  *               [c * chunk, (c + 1) * chunk) of sequence b; chunk must be a
  *               multiple of 32.
@@ -118,12 +123,22 @@ NVJ_API int32_t nvj_paged_decode_whole_sequence_workgroups(int32_t batch, int32_
                                                    int32_t num_kv_heads);
 
 /*
- * Bytes of device workspace nvj_paged_decode_launch needs for the partials
- * (fp32 accumulators plus running max and sum per partial; in balanced mode
- * also batch + 1 int32 prefix sums) for the given `chunk` mode.  Returns 0 on
- * invalid arguments, and for chunk == NVJ_CHUNK_WHOLE_SEQUENCE, which needs none
- * (workspace may then be NULL).
+ * Bytes of device workspace nvj_paged_decode_launch needs for the given `chunk`
+ * mode: the partials (fp32 accumulators plus running max and sum per partial)
+ * and, in balanced mode, in front of them one int32 counter per (sequence, KV
+ * head).  Returns 0 on invalid arguments, and for chunk ==
+ * NVJ_CHUNK_WHOLE_SEQUENCE, which needs none (workspace may then be NULL).  The
+ * balanced size depends on the number of compute units of the current device.
+ *
+ * nvj_paged_decode_counter_bytes: how many bytes at the head of a balanced-split
+ * workspace are its counters (one int32 per (sequence, KV head), padded to 256
+ * bytes; 0 on invalid arguments).  A caller that reuses one workspace for
+ * calls of different shapes needs it: a launch leaves exactly that prefix zero,
+ * what lies behind it holds partials.
  */
+NVJ_API size_t nvj_paged_decode_counter_bytes(int32_t batch, int32_t num_heads,
+                                             int32_t num_kv_heads);
+
 NVJ_API size_t nvj_paged_decode_workspace_bytes(int32_t batch, int32_t num_heads,
                                         int32_t head_dim, int32_t max_blocks,
                                         int32_t block_size, int32_t num_kv_heads,
@@ -145,7 +160,9 @@ NVJ_API size_t nvj_paged_decode_workspace_bytes(int32_t batch, int32_t num_heads
  *                engine/model_runner.py:360)
  *   out          [batch, num_heads, head_dim]                         dtype
  *   workspace    >= nvj_paged_decode_workspace_bytes(...) bytes, 16-byte aligned,
- *                contents need not be initialised
+ *                contents need not be initialised (this entry point clears the
+ *                counters of the balanced split itself, with a small kernel
+ *                ahead of the main one)
  *
  * out[b,h,:] = softmax_{s < ctx[b]}(scale * q[b,h,:] . K[b,s,h/G,:]) V[b,s,h/G,:]
  * with G = num_heads / num_kv_heads, fp32 accumulation, result in `dtype`
@@ -156,9 +173,9 @@ NVJ_API size_t nvj_paged_decode_workspace_bytes(int32_t batch, int32_t num_heads
  * [0, num_blocks); the kernel clamps them into range like the reference (:185)
  * rather than faulting.
  *
- * Two launches on `stream`: the split-K kernel (each workgroup streams its
- * share of positions for all KV heads) and the combine pass; one launch for
- * chunk == NVJ_CHUNK_WHOLE_SEQUENCE.
+ * Launches on `stream`: chunk == 0: the counter-clearing kernel and the
+ * attention kernel; chunk > 0: the split-K kernel and the combine pass; chunk
+ * == NVJ_CHUNK_WHOLE_SEQUENCE: one kernel.
  * Supported: head_dim 128 (every Qwen3 size) or 64 (the reference's toy test
  * shapes), block_size a multiple of 32, chunk a multiple of 32 (0 = balanced
  * split) or NVJ_CHUNK_WHOLE_SEQUENCE.  K/V are read once for up to 16 query
@@ -174,12 +191,19 @@ NVJ_API int nvj_paged_decode_launch(void* stream,
                             int32_t num_blocks, float scale, int32_t chunk, int32_t dtype);
 
 /*
- * The same call with its two launches selectable: NVJ_PHASE_SPLITK runs the
- * split-K kernel only (partials stay in `workspace`), NVJ_PHASE_COMBINE the
- * combine pass only (reads the partials an earlier split-K launch with the
- * same arguments left in `workspace`).  Both bits = nvj_paged_decode_launch.
- * For timing one launch in isolation and for callers that want other work
- * between the two; same reference counterpart as nvj_paged_decode_launch.
+ * The same call with its launches selectable.  NVJ_PHASE_SPLITK: the attention
+ * kernel (all there is for chunk == 0 and NVJ_CHUNK_WHOLE_SEQUENCE; for chunk
+ * > 0 the partials stay in `workspace`).  NVJ_PHASE_COMBINE: the second pass of
+ * the fixed split (reads the partials an earlier split-K launch with the same
+ * arguments left in `workspace`; nothing for the other modes).
+ * NVJ_PHASE_CLEAR_COUNTERS: chunk == 0 only, set the counters at the head of
+ * `workspace` to zero first.  The balanced kernel needs them zero when it
+ * starts and leaves them zero when it ends, so a caller that keeps one
+ * workspace per stream clears it once (this bit alone, or with the first call)
+ * and then passes NVJ_PHASE_SPLITK only: one launch per call.  A workspace whose
+ * counters are not zero gives wrong results (never a fault).  All three bits =
+ * nvj_paged_decode_launch.  Same reference counterpart as
+ * nvj_paged_decode_launch.
  *
  * NVJ_PHASE_VALU_PRODUCTS, or-ed in, runs a measurement variant of the split-K
  * kernel that computes Q.K and P.V with vector-ALU dot products instead of the
@@ -192,6 +216,7 @@ NVJ_API int nvj_paged_decode_launch(void* stream,
 #define NVJ_PHASE_SPLITK  1u
 #define NVJ_PHASE_COMBINE 2u
 #define NVJ_PHASE_VALU_PRODUCTS 4u
+#define NVJ_PHASE_CLEAR_COUNTERS 8u
 NVJ_API int nvj_paged_decode_launch_phases(void* stream,
                             const void* q, const void* k_cache, const void* v_cache,
                             const int32_t* block_tables, const int32_t* context_lens,
@@ -208,20 +233,23 @@ NVJ_API int nvj_paged_decode_launch_phases(void* stream,
  * reference (whose arrays are all allocated by XLA); results are those of
  * nvj_paged_decode_launch(chunk = 0) bit for bit.
  *
- * The split-K partials live in a device array of NVJ_STATIC_SCRATCH_BYTES that is
- * part of the library image: every GPU the library runs on holds its own copy
- * from the first call on that GPU until the process ends.  The call itself
+ * The split-K partials and counters live in a device array of
+ * NVJ_STATIC_SCRATCH_BYTES that is part of the library image: every GPU the
+ * library runs on holds its own copy from the first call on that GPU until the
+ * process ends.  The counters are zero when the library is loaded and every
+ * launch leaves them zero, so the call is a single kernel launch.  The call itself
  * allocates and frees nothing (no hipMalloc / hipFree, no allocating library
  * routine); the first call on a device looks the array's address up once.  The
  * device that `stream` belongs to must be the current device.
  *
- * A problem whose workspace (nvj_paged_decode_workspace_bytes(..., chunk 0))
- * exceeds NVJ_STATIC_SCRATCH_BYTES is rejected with NVJ_ERR_SCRATCH_LIMIT;
- * batch 256 with 32 query heads of 128 dims needs 8.5 MB.  All calls on one GPU
+ * A problem whose partials (nvj_paged_decode_workspace_bytes(..., chunk 0) minus
+ * nvj_paged_decode_counter_bytes) exceed NVJ_STATIC_SCRATCH_BYTES - 64 KiB, or
+ * whose counters exceed 64 KiB (batch * num_kv_heads > 16384), is rejected with
+ * NVJ_ERR_SCRATCH_LIMIT; batch 256 with 32 query heads of 128 dims needs 8.5 MB.  All calls on one GPU
  * share the one array: calls that may overlap in time on the same GPU (two
  * streams, two threads) race on it and must be serialised by the caller; calls
- * on one stream are ordered and safe.  Nothing in the array has to survive from
- * one call to the next.
+ * on one stream are ordered and safe.  Apart from the counters being zero,
+ * nothing in the array has to survive from one call to the next.
  */
 #define NVJ_STATIC_SCRATCH_BYTES (16u << 20)
 NVJ_API int nvj_paged_decode_static_launch(void* stream,

@@ -29,6 +29,7 @@ SYMBOLS = {
     "nvj_paged_decode_default_chunk": (_c.c_int32, [_c.c_int32] * 4),
     "nvj_paged_decode_whole_sequence_workgroups": (_c.c_int32, [_c.c_int32] * 3),
     "nvj_paged_decode_workspace_bytes": (_c.c_size_t, [_c.c_int32] * 7),
+    "nvj_paged_decode_counter_bytes": (_c.c_size_t, [_c.c_int32] * 3),
     "nvj_paged_decode_launch": (_c.c_int, [
         _c.c_void_p, _c.c_void_p, _c.c_void_p, _c.c_void_p, _c.c_void_p, _c.c_void_p,
         _c.c_void_p, _c.c_void_p, _c.c_size_t,
@@ -65,9 +66,11 @@ SYMBOLS = {
 NVJ_CHUNK_WHOLE_SEQUENCE = -1
 NVJ_STATIC_SCRATCH_BYTES = 16 << 20
 NVJ_ERR_SCRATCH_LIMIT = -7
+NVJ_ERR_ALIGNMENT = -8
 NVJ_PHASE_SPLITK = 1
 NVJ_PHASE_COMBINE = 2
 NVJ_PHASE_VALU_PRODUCTS = 4
+NVJ_PHASE_CLEAR_COUNTERS = 8
 
 _lock = threading.Lock()
 _lib = None

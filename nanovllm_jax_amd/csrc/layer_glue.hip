@@ -180,7 +180,7 @@ extern "C" int nvj_add_rms_norm_launch(void* stream, const void* x, const void* 
   if ((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(residual) |
        reinterpret_cast<uintptr_t>(weight) | reinterpret_cast<uintptr_t>(y) |
        reinterpret_cast<uintptr_t>(residual_out)) & 15u)
-    return NVJ_ERR_BAD_SHAPE;
+    return NVJ_ERR_ALIGNMENT;
   const int row_pieces = hidden / 8;
   const int per_lane = (row_pieces + 63) / 64;
   const auto s = static_cast<hipStream_t>(stream);
@@ -204,7 +204,7 @@ extern "C" int nvj_silu_and_mul_launch(void* stream, const void* x, int64_t x_ro
   if (num_tokens == 0) return NVJ_OK;
   if (!x || !y) return NVJ_ERR_NULL_POINTER;
   if ((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(y)) & 15u)
-    return NVJ_ERR_BAD_SHAPE;
+    return NVJ_ERR_ALIGNMENT;
   const int out_pieces = intermediate / 8;
   const int64_t blocks = ((int64_t)num_tokens * out_pieces + 255) / 256;
   if (blocks > INT32_MAX) return NVJ_ERR_BAD_SHAPE;

@@ -689,13 +689,15 @@ __device__ __forceinline__ void write_output(const DecodeArgs& a, int b, int kvh
   }
 }
 
-// Unnormalised partial (D f32 per head) + (max, sum) to slot `slot` of the workspace.
+// Unnormalised partial (D f32 per head) + (max, sum) to the workspace.  A
+// partial record is D + 2 floats of one query head; `rec_base` is the record of
+// the first query head of this wave's KV head.
 template <int D>
-__device__ __forceinline__ void write_partial(const DecodeArgs& a, int64_t slot, int kvh, int lane,
+__device__ __forceinline__ void write_partial(const DecodeArgs& a, int64_t rec_base, int lane,
                                               const f32x4 (&acc)[8], float m_run, float l_run) {
   const int r = lane & 15, kg = lane >> 4;
   if (r >= a.group || 32 * kg >= D) return;
-  const int64_t row = slot * a.num_heads + kvh * a.group + r;
+  const int64_t row = rec_base + r;
   float4* prow = reinterpret_cast<float4*>(a.part_o + row * D + 32 * kg);
 #pragma unroll
   for (int e = 0; e < 4; ++e) {
@@ -705,23 +707,9 @@ __device__ __forceinline__ void write_partial(const DecodeArgs& a, int64_t slot,
   if (kg == 0) reinterpret_cast<float2*>(a.part_ml)[row] = make_float2(m_run, l_run);
 }
 
-// compute_segment, then: `direct` (the segment is the whole sequence) -> out,
-// otherwise -> partial slot `slot`.
-template <int D, bool F16, int VG = 0>
-__device__ __forceinline__ void run_segment(const DecodeArgs& a, uint4* lds, int b, int kvh,
-                                            int t0, int t1, int64_t slot, bool direct,
-                                            int lane) {
-  f32x4 acc[8];
-  float m_run, l_run;
-  if constexpr (VG > 0) compute_segment_valu<VG>(a, lds, b, kvh, t0, t1, lane, acc, m_run, l_run);
-  else compute_segment<D, F16>(a, lds, b, kvh, t0, t1, lane, acc, m_run, l_run);
-  if (direct) write_output<D, F16>(a, b, kvh, lane, acc, l_run);
-  else write_partial<D>(a, slot, kvh, lane, acc, m_run, l_run);
-}
-
 // Fixed-chunk split: grid.x = batch * max_chunks, grid.y = num_kv_heads / NW,
 // block = NW * 64.  Workgroup (b, c) owns positions [c*chunk, (c+1)*chunk) of
-// sequence b; partial slot = b * max_chunks + c.
+// sequence b; partial slot = b * max_chunks + c holds all query heads.
 template <int NW, int D, bool F16>
 __global__ __launch_bounds__(NW * 64) void paged_decode_splitk_kernel(DecodeArgs a, int chunk,
                                                                       int max_chunks) {
@@ -735,9 +723,13 @@ __global__ __launch_bounds__(NW * 64) void paged_decode_splitk_kernel(DecodeArgs
   const int t0 = c * chunk;
   if (t0 >= ctx) return;  // also every chunk of an empty sequence
   const int t1 = min(ctx, t0 + chunk);
-  const bool direct = ctx <= chunk;
-  run_segment<D, F16>(a, k_tile[wave], b, blockIdx.y * NW + wave, t0, t1,
-                      (int64_t)b * max_chunks + c, direct, lane);
+  const int kvh = blockIdx.y * NW + wave;
+  f32x4 acc[8];
+  float m_run, l_run;
+  compute_segment<D, F16>(a, k_tile[wave], b, kvh, t0, t1, lane, acc, m_run, l_run);
+  if (ctx <= chunk) write_output<D, F16>(a, b, kvh, lane, acc, l_run);
+  else write_partial<D>(a, ((int64_t)b * max_chunks + c) * a.num_heads + kvh * a.group, lane, acc,
+                        m_run, l_run);
 }
 
 // Whole-sequence split: every sequence is finished inside one workgroup, so
@@ -832,35 +824,257 @@ __device__ __forceinline__ int wave_inclusive_scan(int x) {
   return x;
 }
 
-// Balanced split: the 32-position steps of all sequences, laid end to end in
-// batch order, are cut into `num_wgs` equal runs of `S` steps (at least
-// `min_steps`); workgroup g owns steps [g*S, (g+1)*S) whatever sequences they
-// belong to.  A run that crosses a sequence boundary is processed as one
-// segment per sequence.  The segment of (workgroup g, sequence b) uses partial
-// slot g + b, which is unique because g and b only grow along the runs; the
-// slots of one sequence are consecutive.  Every workgroup derives the cut from
-// context_lens itself (a wave-wide prefix sum over the batch), so the host
-// never needs the lengths.  Workgroup 0 also leaves the exclusive prefix sums
-// (steps before each sequence, total at [batch]) in `prefix` for the combine
-// pass.  grid.x = num_wgs, grid.y = num_kv_heads / NW, block = NW * 64.
-template <int NW, int D, bool F16, int VG = 0>
-__global__ __launch_bounds__(NW * 64) void paged_decode_balanced_kernel(DecodeArgs a, int batch,
-                                                                        int num_wgs,
-                                                                        int min_steps,
-                                                                        int32_t* prefix) {
-  __shared__ uint4 k_tile[NW][kStep * HeadDim<D>::kLdsRowPieces];
+// ---------------------------------------------------------------------------
+// Balanced split: one launch for any mix of lengths.
+//
+// A workgroup is 8 waves = `hpw` KV heads x R = 8 / hpw parts (hpw is the
+// largest of 8, 4, 2, 1 that still leaves one row per CU, see the host side).
+// The unit of work is a "row step": one 32-position step of one row, a row
+// being (sequence b, head group hg of hpw KV heads).  All row steps, ordered
+// by (b, hg, step), form one axis of length T = (num_kv_heads / hpw) * sum of
+// steps.  The axis is cut into sub-runs of `lp` row steps, lp the same for
+// all: sub-run j = [j*lp, (j+1)*lp) belongs to workgroup j / R, part j % R, and
+// is walked by the hpw waves of that part, one KV head each.  Every wave
+// derives the cut from context_lens itself (a wave-wide prefix sum over the
+// batch), so the host never needs the lengths.
+//
+// A sub-run that covers a whole row writes the output directly.  Otherwise a
+// row is shared by several sub-runs; the piece of row `row` in sub-run j is a
+// segment and owns partial slot j + row (unique, because j and row only grow
+// along the axis, and consecutive within a row).  When the whole run of a
+// workgroup lies inside one row, its parts are first merged through LDS (a
+// wave's K tile is free by then) and part 0 writes one partial for all of
+// them; the other parts mark their slots empty (sum 0).
+//
+// Merge without a second launch: `counters` holds one int32 per (sequence, KV
+// head), zero between launches.  A wave that has written partials for a row
+// adds the number of sub-runs they stand for; the wave whose addition
+// completes the row's count (the number of sub-runs that touch the row, known
+// from the cut) merges the row's partials in slot order, writes the output and
+// puts the counter back to zero.  Nothing ever waits for another workgroup.
+// ---------------------------------------------------------------------------
+
+// Record (see write_partial) of query head 0 of KV head `h_in_row` of a slot.
+__device__ __forceinline__ int64_t balanced_record(const DecodeArgs& a, int64_t slot, int hpw,
+                                                   int h_in_row) {
+  return (slot * hpw + h_in_row) * a.group;
+}
+
+// Partials of the balanced split travel between workgroups of one launch, and
+// workgroups on different XCDs do not share an L2.  They are therefore written
+// and read with device-scope accesses (cache policy sc1: written through to,
+// and read from, the point where the XCDs meet), ordered against the row's
+// counter by waiting for the stores to be acknowledged.  No cache-wide
+// write-back or invalidate is ever issued; those stall the K/V stream of every
+// other wave on the XCD.  The accesses are 16-byte buffer instructions over a
+// window that starts at a wave-uniform address.
+//
+// Layout of the partial of one (slot, KV head), chosen so that every store
+// instruction of a wave writes one contiguous run: 16-byte piece i (0..7) of
+// lane (r = query head, kg = dim group) sits at piece index
+// i * (D/32 * G) + kg * G + r.  Piece 2e holds acc[0..3][e], piece 2e+1
+// acc[4..7][e] of that lane.  The (max, sum) pairs follow the record order.
+typedef __attribute__((ext_vector_type(4))) float vfloat4;
+typedef __attribute__((ext_vector_type(2))) float vfloat2;
+typedef __attribute__((ext_vector_type(4))) unsigned int vuint4;
+typedef __attribute__((ext_vector_type(2))) unsigned int vuint2;
+constexpr int kDeviceScope = 16;   // buffer cache policy: sc1
+
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t device_window(const void* base, int64_t bytes) {
+  const int n = (int)(bytes < 0x7fffffff ? bytes : 0x7fffffff);
+  return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, n, 0x00020000);
+}
+
+template <int D>
+__device__ __forceinline__ void write_partial_coherent(const DecodeArgs& a, int64_t rec_base,
+                                                       int lane, const f32x4 (&acc)[8],
+                                                       float m_run, float l_run) {
+  constexpr int KG = D / 32;
+  const int r = lane & 15, kg = lane >> 4;
+  if (r >= a.group || kg >= KG) return;
+  const __amdgpu_buffer_rsrc_t wo =
+      device_window(a.part_o + rec_base * D, (int64_t)a.group * D * sizeof(float));
+  const int lane_off = (kg * a.group + r) * 16, piece_stride = KG * a.group * 16;
+#pragma unroll
+  for (int e = 0; e < 4; ++e) {
+    const vfloat4 lo = {acc[0][e], acc[1][e], acc[2][e], acc[3][e]};
+    const vfloat4 hi = {acc[4][e], acc[5][e], acc[6][e], acc[7][e]};
+    __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(vuint4, lo), wo,
+                                           lane_off + 2 * e * piece_stride, 0, kDeviceScope);
+    __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(vuint4, hi), wo,
+                                           lane_off + (2 * e + 1) * piece_stride, 0, kDeviceScope);
+  }
+  if (kg == 0) {
+    const __amdgpu_buffer_rsrc_t wm =
+        device_window(a.part_ml + rec_base * 2, (int64_t)a.group * 2 * sizeof(float));
+    const vfloat2 ml = {m_run, l_run};
+    __builtin_amdgcn_raw_buffer_store_b64(__builtin_bit_cast(vuint2, ml), wm, r * 8, 0,
+                                          kDeviceScope);
+  }
+}
+
+// All earlier stores of this wave have been acknowledged (and no later memory
+// operation is moved ahead of this point by the compiler).
+__device__ __forceinline__ void wait_for_stores() {
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+}
+
+// arrive: the wave has written its partials of row [r0, r1) (row steps on the
+// axis) of (sequence b, KV head kvh), standing for `n` sub-runs, and publishes
+// them.  merge_row: all partials of the row are there; merge them in slot order
+// and write the output.  `lds` is the wave's own tile (free at that point).
+//
+// The merge keeps the chain of dependent memory round trips short: the (max,
+// sum) pairs of 16 slots are fetched by four loads issued together and spread
+// to the lanes through LDS; empty slots are then skipped, and the accumulators
+// of two real partials are in flight at once.
+// Returns true when this arrival completed the row: the caller then owes the
+// row its merge (merge_row), at a time of its choosing.
+__device__ __forceinline__ bool arrive(const DecodeArgs& a, int32_t* counters, int b, int kvh,
+                                       int r0, int r1, int lp, int n, int lane) {
+  // the partial stores of every lane have reached the device before the count does
+  wait_for_stores();
+  int32_t* counter = counters + (int64_t)b * a.num_kv_heads + kvh;
+  int old = 0;
+  if (lane == 0)
+    old = __hip_atomic_fetch_add(counter, n, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  old = __builtin_amdgcn_readfirstlane(old);
+  const int expected = (r1 - 1) / lp - r0 / lp + 1;
+  if (old + n != expected) return false;
+  // last to arrive: every other partial of the row was acknowledged before its
+  // writer's count, which this wave has just seen
+  asm volatile("" ::: "memory");
+  if (lane == 0) __hip_atomic_store(counter, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  return true;
+}
+
+template <int D, bool F16>
+__device__ __forceinline__ void merge_row(const DecodeArgs& a, uint4* lds, int b, int kvh,
+                                          int hpw, int r0, int r1, int lp, int lane) {
+  const int first = r0 / lp;
+  const int expected = (r1 - 1) / lp - first + 1;
+  const int hg = kvh / hpw;
+  const int rows_per_seq = a.num_kv_heads / hpw;
+  const int64_t slot0 = (int64_t)first + (int64_t)b * rows_per_seq + hg;
+  // lanes of padding heads / padding dims read a real record and drop it later
+  const int r = min(lane & 15, a.group - 1);
+  const int kg = (32 * (lane >> 4) < D) ? (lane >> 4) : 0;
+  constexpr int KG = D / 32;
+  const int64_t rec0 = balanced_record(a, slot0, hpw, kvh - hg * hpw);   // slot0, head 0
+  const int64_t rec_stride = (int64_t)hpw * a.group;                     // per slot
+  const __amdgpu_buffer_rsrc_t wm = device_window(
+      a.part_ml + rec0 * 2, ((int64_t)(expected - 1) * rec_stride + a.group) * 2 * sizeof(float));
+  const int lane_off = (kg * a.group + r) * 16, piece_stride = KG * a.group * 16;
+  vfloat2* lds_ml = reinterpret_cast<vfloat2*>(lds);   // [16 slots][16 heads]
+  f32x4 acc[8];
+#pragma unroll
+  for (int jd = 0; jd < 8; ++jd) acc[jd] = f32x4{0.f, 0.f, 0.f, 0.f};
+  float m_run = kNegBig, l_run = 0.f;
+  for (int base = 0; base < expected; base += 16) {
+    // (max, sum) of slots base .. base + 15 for the 16 head columns: lane (r, kg)
+    // fetches slot base + 4 * i + kg for i = 0 .. 3; slots past the end repeat the last
+    vfloat2 got[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int s = min(base + 4 * i + (lane >> 4), expected - 1);
+      got[i] = __builtin_bit_cast(vfloat2, __builtin_amdgcn_raw_buffer_load_b64(
+                                               wm, (int)((s * rec_stride + r) * 8), 0, kDeviceScope));
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i) lds_ml[(4 * i + (lane >> 4)) * 16 + (lane & 15)] = got[i];
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    const int count = min(16, expected - base);
+    // which of the slots hold a partial (sum > 0): the same for every head
+    uint32_t real = 0;
+    float m_chunk = kNegBig;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+      const vfloat2 x = lds_ml[i * 16 + (lane & 15)];
+      if (i < count && x.y > 0.f) {
+        real |= 1u << i;
+        m_chunk = fmaxf(m_chunk, x.x);
+      }
+    }
+    real = __builtin_amdgcn_readfirstlane(real);
+    if (real != 0u) {
+      const float m_new = fmaxf(m_run, m_chunk);
+      const float keep = __builtin_amdgcn_exp2f((m_run - m_new) * a.scale_log2e);
+      m_run = m_new;
+      l_run *= keep;
+#pragma unroll
+      for (int jd = 0; jd < 8; ++jd) acc[jd] *= keep;
+      while (real != 0u) {
+        // two real partials at a time; an absent second repeats the first with weight 0
+        const int i0 = __builtin_ctz(real);
+        real &= real - 1u;
+        const bool two = real != 0u;
+        const int i1 = two ? __builtin_ctz(real) : i0;
+        if (two) real &= real - 1u;
+        const __amdgpu_buffer_rsrc_t win0 = device_window(
+            a.part_o + (rec0 + (base + i0) * rec_stride) * D, (int64_t)a.group * D * sizeof(float));
+        const __amdgpu_buffer_rsrc_t win1 = device_window(
+            a.part_o + (rec0 + (base + i1) * rec_stride) * D, (int64_t)a.group * D * sizeof(float));
+        vfloat4 v0[8], v1[8];
+#pragma unroll
+        for (int i = 0; i < 8; ++i)
+          v0[i] = __builtin_bit_cast(vfloat4, __builtin_amdgcn_raw_buffer_load_b128(
+                                                  win0, lane_off + i * piece_stride, 0, kDeviceScope));
+#pragma unroll
+        for (int i = 0; i < 8; ++i)
+          v1[i] = __builtin_bit_cast(vfloat4, __builtin_amdgcn_raw_buffer_load_b128(
+                                                  win1, lane_off + i * piece_stride, 0, kDeviceScope));
+        const vfloat2 ml0 = lds_ml[i0 * 16 + (lane & 15)];
+        const vfloat2 ml1 = lds_ml[i1 * 16 + (lane & 15)];
+        const float w0 = __builtin_amdgcn_exp2f((ml0.x - m_new) * a.scale_log2e);
+        const float w1 = two ? __builtin_amdgcn_exp2f((ml1.x - m_new) * a.scale_log2e) : 0.f;
+        l_run = fmaf(w0, ml0.y, fmaf(w1, ml1.y, l_run));
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          acc[0][e] = fmaf(w0, v0[2 * e].x, fmaf(w1, v1[2 * e].x, acc[0][e]));
+          acc[1][e] = fmaf(w0, v0[2 * e].y, fmaf(w1, v1[2 * e].y, acc[1][e]));
+          acc[2][e] = fmaf(w0, v0[2 * e].z, fmaf(w1, v1[2 * e].z, acc[2][e]));
+          acc[3][e] = fmaf(w0, v0[2 * e].w, fmaf(w1, v1[2 * e].w, acc[3][e]));
+          acc[4][e] = fmaf(w0, v0[2 * e + 1].x, fmaf(w1, v1[2 * e + 1].x, acc[4][e]));
+          acc[5][e] = fmaf(w0, v0[2 * e + 1].y, fmaf(w1, v1[2 * e + 1].y, acc[5][e]));
+          acc[6][e] = fmaf(w0, v0[2 * e + 1].z, fmaf(w1, v1[2 * e + 1].z, acc[6][e]));
+          acc[7][e] = fmaf(w0, v0[2 * e + 1].w, fmaf(w1, v1[2 * e + 1].w, acc[7][e]));
+        }
+      }
+    }
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();   // the next chunk overwrites lds_ml
+  }
+  write_output<D, F16>(a, b, kvh, lane, acc, l_run);
+}
+
+// grid.x = num_wgs, block = 512.  `min_steps`: lower bound of lp.
+template <int D, bool F16, int VG = 0>
+__global__ __launch_bounds__(512) void paged_decode_balanced_kernel(DecodeArgs a, int batch,
+                                                                    int num_wgs, int min_steps,
+                                                                    int hpw, int32_t* counters) {
+  using H = HeadDim<D>;
+  constexpr int NW = 8;
+  __shared__ uint4 k_tile[NW][kStep * H::kLdsRowPieces];
+  constexpr int kLanesWithDims = D / 32 * 16;   // lanes whose k-group holds real dims
+  static_assert(sizeof(uint4) * kStep * H::kLdsRowPieces >= 34 * kLanesWithDims * sizeof(float),
+                "a wave's K tile must hold its partial");
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int lane = threadIdx.x & 63;
   const int g = blockIdx.x;
   const int cap = a.max_blocks * a.block_size;
-  const bool writer = g == 0 && blockIdx.y == 0 && wave == 0;
+  const int parts = NW / hpw;
+  const int rows_per_seq = a.num_kv_heads / hpw;
+  const int part = wave / hpw;
+  const int h_in_row = wave - part * hpw;
 
   auto ctx_of = [&](int idx) { return idx < batch ? min(max(a.context_lens[idx], 0), cap) : 0; };
   auto steps_of = [&](int idx) { return (ctx_of(idx) + kStep - 1) / kStep; };
 
   // One pass over the batch, 64 sequences at a time: total number of steps,
-  // and for the first kKeep groups the per-lane (steps, steps before) pairs are
-  // kept so that locating the start below needs no second read.
+  // and for the first kKeep groups the per-lane (length, steps before) pairs
+  // are kept so that locating a position below needs no second read.
   constexpr int kKeep = 4;
   int kept_ctx[kKeep], kept_excl[kKeep];
 #pragma unroll
@@ -873,113 +1087,251 @@ __global__ __launch_bounds__(NW * 64) void paged_decode_balanced_kernel(DecodeAr
       const int n = (kept_ctx[k] + kStep - 1) / kStep;
       const int incl = wave_inclusive_scan(n);
       kept_excl[k] = total + incl - n;
-      if (writer && k * 64 + lane < batch) prefix[k * 64 + lane] = kept_excl[k];
       total += __builtin_amdgcn_readlane(incl, 63);
     }
   }
   total_kept = total;
   for (int base = kKeep * 64; base < batch; base += 64) {
     const int n = steps_of(base + lane);
-    const int incl = wave_inclusive_scan(n);
-    if (writer && base + lane < batch) prefix[base + lane] = total + incl - n;
-    total += __builtin_amdgcn_readlane(incl, 63);
+    total += __builtin_amdgcn_readlane(wave_inclusive_scan(n), 63);
   }
-  if (writer && lane == 0) prefix[batch] = total;
-  const int run = max((total + num_wgs - 1) / num_wgs, min_steps);
-  const int start = g * run;
-  if (start >= total) return;
-  const int end = min(total, start + run);
-
-  // the sequence that holds step `start`, the steps before it and its length
-  int b = batch, before = total, first_ctx = -1;
-  bool found = false;
+  // No step belongs to an empty sequence: its output row (zeros, 0 / (0 + 1e-9))
+  // is written here, sequence b by workgroup b modulo the grid.  The lengths of
+  // the first kKeep * 64 sequences are in registers already.
+  for (int b = g; b < batch; b += gridDim.x) {
+    int c;
+    if (b < kKeep * 64) {
+      int mine = kept_ctx[0];
 #pragma unroll
-  for (int k = 0; k < kKeep; ++k) {
-    const int n = (kept_ctx[k] + kStep - 1) / kStep;
-    const unsigned long long hit =
-        __ballot(!found && n > 0 && kept_excl[k] <= start && start < kept_excl[k] + n);
-    if (hit != 0ull) {
-      const int src = __builtin_ctzll(hit);
-      b = k * 64 + src;
-      before = __shfl(kept_excl[k], src, 64);
-      first_ctx = __shfl(kept_ctx[k], src, 64);
-      found = true;
+      for (int k = 1; k < kKeep; ++k) mine = (b >> 6) == k ? kept_ctx[k] : mine;
+      c = __shfl(mine, b & 63, 64);
+    } else {
+      c = min(as_constant(a.context_lens)[b], cap);
+    }
+    if (__builtin_amdgcn_readfirstlane(c) <= 0) {
+      uint4* orow = a.out + (int64_t)b * a.num_heads * H::kPieces;
+      for (int i = threadIdx.x; i < a.num_heads * H::kPieces; i += NW * 64)
+        orow[i] = make_uint4(0u, 0u, 0u, 0u);
     }
   }
-  if (!found) {
-    int running = total_kept;
-    for (int base = kKeep * 64; base < batch; base += 64) {
-      const int n = steps_of(base + lane);
-      const int incl = wave_inclusive_scan(n);
-      const int excl = running + incl - n;
-      const unsigned long long hit = __ballot(n > 0 && excl <= start && start < excl + n);
+  const int axis = rows_per_seq * total;   // T
+  const int lp = max(((axis + num_wgs - 1) / num_wgs + parts - 1) / parts, min_steps);
+  const int run = lp * parts;
+  const int start = g * run;
+  if (start >= axis) return;
+  const int end = min(axis, start + run);
+
+  // the sequence whose rows hold axis position x: its index, the steps before
+  // it and its length (all wave-uniform)
+  auto locate = [&](int x, int& b, int& before, int& ctx) {
+    b = batch; before = total; ctx = 0;
+    bool found = false;
+#pragma unroll
+    for (int k = 0; k < kKeep; ++k) {
+      const int n = (kept_ctx[k] + kStep - 1) / kStep;
+      const int lo = rows_per_seq * kept_excl[k];
+      const unsigned long long hit =
+          __ballot(!found && n > 0 && lo <= x && x < lo + rows_per_seq * n);
       if (hit != 0ull) {
         const int src = __builtin_ctzll(hit);
-        b = base + src;
-        before = __shfl(excl, src, 64);
-        break;
+        b = k * 64 + src;
+        before = __shfl(kept_excl[k], src, 64);
+        ctx = __shfl(kept_ctx[k], src, 64);
+        found = true;
       }
-      running += __builtin_amdgcn_readlane(incl, 63);
+    }
+    if (!found) {
+      int running = total_kept;
+      for (int base = kKeep * 64; base < batch; base += 64) {
+        const int c = ctx_of(base + lane);
+        const int n = (c + kStep - 1) / kStep;
+        const int incl = wave_inclusive_scan(n);
+        const int lo = rows_per_seq * (running + incl - n);
+        const unsigned long long hit = __ballot(n > 0 && lo <= x && x < lo + rows_per_seq * n);
+        if (hit != 0ull) {
+          const int src = __builtin_ctzll(hit);
+          b = base + src;
+          before = __shfl(running + incl - n, src, 64);
+          ctx = __shfl(c, src, 64);
+          break;
+        }
+        running += __builtin_amdgcn_readlane(incl, 63);
+      }
+    }
+    b = __builtin_amdgcn_readfirstlane(b);
+    before = __builtin_amdgcn_readfirstlane(before);
+    ctx = __builtin_amdgcn_readfirstlane(ctx);
+  };
+
+  int b0, before0, ctx0;
+  locate(start, b0, before0, ctx0);
+  if (b0 >= batch || ctx0 <= 0) return;   // cannot happen when the prefix sums are right
+  const int nb0 = (ctx0 + kStep - 1) / kStep;
+  const int hg0 = (start - rows_per_seq * before0) / nb0;
+  const int row0 = rows_per_seq * before0 + hg0 * nb0;   // axis position of the row's step 0
+  const int xs = start + part * lp;
+  const int xe = min(end, xs + lp);
+  const int64_t subrun = (int64_t)g * parts + part;
+  // Does the whole run of the workgroup lie inside one row?  Then every wave has
+  // at most one segment, and the parts of a head meet in LDS before anything is
+  // written.  Otherwise every wave walks its own sub-run across the rows.
+  const bool single = end <= row0 + nb0;
+  const int nparts = (end - start + lp - 1) / lp;   // parts of this workgroup that have work
+  if (!single && xs >= xe) return;
+
+  int b = b0, before = before0, ctx = ctx0;
+  if (!single && part > 0) locate(xs, b, before, ctx);
+  // Every quantity of the walk is wave-uniform; readfirstlane says so, so that
+  // lengths, page lookups and address arithmetic stay on the scalar unit.  The
+  // guards (b inside the batch, x not before the sequence) cannot fire when
+  // the prefix sums are right; they keep every index in range regardless.
+  if (single && part > 0 && xs < xe && !(start == row0 && end == row0 + nb0)) {
+    // Part 0 will carry this part's share in its own partial: this part's slot
+    // is marked empty (sum 0).  Stored now, so that the acknowledgement it must
+    // wait for before the parts meet arrives while the wave works.
+    if (lane < a.group) {
+      const int64_t rec =
+          balanced_record(a, subrun + (int64_t)b0 * rows_per_seq + hg0, hpw, h_in_row);
+      const __amdgpu_buffer_rsrc_t wm =
+          device_window(a.part_ml + rec * 2, (int64_t)a.group * 2 * sizeof(float));
+      const vfloat2 empty = {kNegBig, 0.f};
+      __builtin_amdgcn_raw_buffer_store_b64(__builtin_bit_cast(vuint2, empty), wm, lane * 8, 0,
+                                            kDeviceScope);
     }
   }
-  b = __builtin_amdgcn_readfirstlane(b);
-  before = __builtin_amdgcn_readfirstlane(before);
-  first_ctx = __builtin_amdgcn_readfirstlane(first_ctx);
-
-  // Walk the run.  The guards (b inside the batch, pos not before the
-  // sequence) cannot fire when the prefix sums are right; they keep every
-  // index in range regardless.
-  // Every quantity of the walk is wave-uniform; readfirstlane says so, so
-  // that lengths, page lookups and address arithmetic stay on the scalar unit.
-  int pos = start;
-  while (pos < end && b < batch && pos >= before) {
-    const int sb = __builtin_amdgcn_readfirstlane(b);
-    // the first sequence's length is already in registers from the scan
-    const int ctx = __builtin_amdgcn_readfirstlane(
-        first_ctx >= 0 ? first_ctx : min(max(as_constant(a.context_lens)[sb], 0), cap));
-    first_ctx = -1;
-    const int nb = (ctx + kStep - 1) / kStep;
-    if (pos >= before + nb) {  // empty sequence, or this one is finished
-      before += nb;
-      b = sb + 1;
-      continue;
+  int x = xs;
+  int owed = 0, owed_b[2] = {0, 0}, owed_kvh[2] = {0, 0}, owed_row[2] = {0, 0}, owed_nb[2] = {1, 1};
+  for (;;) {
+    // ---- the next segment of this wave's sub-run: row (sb, hg), steps [st, en) ----
+    int sb = 0, hg = 0, nb = 1, row = 0, st = 0, en = 0;
+    bool have = false;
+    while (x < xe && b < batch) {
+      sb = __builtin_amdgcn_readfirstlane(b);
+      nb = (ctx + kStep - 1) / kStep;
+      const int seq0 = rows_per_seq * before;
+      if (x < seq0) break;
+      if (nb == 0 || x >= seq0 + rows_per_seq * nb) {  // empty sequence, or this one is finished
+        before += nb;
+        b = sb + 1;
+        ctx = b < batch ? __builtin_amdgcn_readfirstlane(
+                              min(max(as_constant(a.context_lens)[b], 0), cap))
+                        : 0;
+        continue;
+      }
+      hg = (x - seq0) / nb;
+      row = seq0 + hg * nb;
+      st = x - row;
+      en = min(nb, st + (xe - x));
+      have = true;
+      break;
     }
-    const int seg_end = min(end, before + nb);
-    const int t0 = __builtin_amdgcn_readfirstlane((pos - before) * kStep);
-    const int t1 = __builtin_amdgcn_readfirstlane(min(ctx, (seg_end - before) * kStep));
-    const bool direct = pos == before && seg_end == before + nb;
-    run_segment<D, F16, VG>(a, k_tile[wave], sb, blockIdx.y * NW + wave, t0, t1,
-                            (int64_t)(g + sb), direct, lane);
-    pos = seg_end;
+    if (!have && !single) break;
+    const int kvh = (single ? hg0 : hg) * hpw + h_in_row;
+    f32x4 acc[8];
+#pragma unroll
+    for (int jd = 0; jd < 8; ++jd) acc[jd] = f32x4{0.f, 0.f, 0.f, 0.f};
+    float m_run = kNegBig, l_run = 0.f;
+    if (have) {
+      const int t0 = __builtin_amdgcn_readfirstlane(st * kStep);
+      const int t1 = __builtin_amdgcn_readfirstlane(min(ctx, en * kStep));
+      if constexpr (VG > 0)
+        compute_segment_valu<VG>(a, k_tile[wave], sb, kvh, t0, t1, lane, acc, m_run, l_run);
+      else
+        compute_segment<D, F16>(a, k_tile[wave], sb, kvh, t0, t1, lane, acc, m_run, l_run);
+      x += en - st;
+    }
+
+    bool direct = st == 0 && en == nb;   // the segment is the whole row
+    int covers = 1;                      // sub-runs this wave's partial stands for
+    if (single) {
+      sb = b0; hg = hg0; nb = nb0; row = row0;
+      direct = start == row0 && end == row0 + nb0;
+      covers = nparts;
+      if (nparts > 1) {
+        const bool holds_dims = lane < kLanesWithDims;
+        if (part > 0 && have) {
+          // value v of lane l at float v * kLanesWithDims + l of the wave's own tile
+          if (holds_dims) {
+            float* mine = reinterpret_cast<float*>(k_tile[wave]) + lane;
+#pragma unroll
+            for (int jd = 0; jd < 8; ++jd)
+#pragma unroll
+              for (int e = 0; e < 4; ++e) mine[(4 * jd + e) * kLanesWithDims] = acc[jd][e];
+            mine[32 * kLanesWithDims] = m_run;
+            mine[33 * kLanesWithDims] = l_run;
+          }
+          // the empty marker stored before the work began has been acknowledged
+          // by now; part 0 publishes the count after the barrier below
+          if (!direct) wait_for_stores();
+        }
+        __syncthreads();
+        if (part > 0) return;
+        if (holds_dims) {
+          for (int p = 1; p < nparts; ++p) {
+            const float* theirs = reinterpret_cast<const float*>(k_tile[wave + p * hpw]) + lane;
+            const float m_p = theirs[32 * kLanesWithDims], l_p = theirs[33 * kLanesWithDims];
+            const float m_new = fmaxf(m_run, m_p);
+            const float keep = __builtin_amdgcn_exp2f((m_run - m_new) * a.scale_log2e);
+            const float w = __builtin_amdgcn_exp2f((m_p - m_new) * a.scale_log2e);
+            m_run = m_new;
+            l_run = fmaf(l_run, keep, w * l_p);
+#pragma unroll
+            for (int jd = 0; jd < 8; ++jd)
+#pragma unroll
+              for (int e = 0; e < 4; ++e)
+                acc[jd][e] = fmaf(acc[jd][e], keep, w * theirs[(4 * jd + e) * kLanesWithDims]);
+          }
+        }
+      }
+      if (part > 0) return;
+    }
+
+    if (direct) {
+      write_output<D, F16>(a, sb, kvh, lane, acc, l_run);
+    } else {
+      const int64_t slot = subrun + (int64_t)sb * rows_per_seq + hg;
+      write_partial_coherent<D>(a, balanced_record(a, slot, hpw, h_in_row), lane, acc, m_run,
+                                l_run);
+      if (arrive(a, counters, sb, kvh, row, row + nb, lp, covers, lane)) {
+        // at most the first and the last segment of a sub-run are not whole rows
+        if (owed == 0) { owed_b[0] = sb; owed_kvh[0] = kvh; owed_row[0] = row; owed_nb[0] = nb; }
+        else { owed_b[1] = sb; owed_kvh[1] = kvh; owed_row[1] = row; owed_nb[1] = nb; }
+        ++owed;
+      }
+    }
+    if (single) break;
+  }
+  // the merges this wave owes, after its own work
+  for (int i = 0; i < owed; ++i) {
+    const int ob = __builtin_amdgcn_readfirstlane(i == 0 ? owed_b[0] : owed_b[1]);
+    const int okvh = __builtin_amdgcn_readfirstlane(i == 0 ? owed_kvh[0] : owed_kvh[1]);
+    const int orow = __builtin_amdgcn_readfirstlane(i == 0 ? owed_row[0] : owed_row[1]);
+    const int onb = __builtin_amdgcn_readfirstlane(i == 0 ? owed_nb[0] : owed_nb[1]);
+    merge_row<D, F16>(a, k_tile[wave], ob, okvh, hpw, orow, orow + onb, lp, lane);
   }
 }
 
-// Merge the partials of one (sequence, query head).  grid = (B, Hq), block = 128
-// lanes, one per output dim.  Fixed-chunk mode (prefix == nullptr): the
-// partials of sequence b are slots b*max_chunks .. + ceil(ctx/chunk).  Balanced
-// mode: they are slots g_first + b .. g_last + b, where g_first..g_last are the
-// workgroups whose runs of `run` steps touch the sequence.  A sequence with one
-// partial was written by the split kernel itself; an empty one gives zeros.
+// Sets n int32 to zero (the counters of the balanced split; a kernel, not a
+// memset, so that the launch can be recorded into a graph).
+__global__ __launch_bounds__(256) void zero_int32_kernel(int32_t* p, int n) {
+  const int i = blockIdx.x * 256 + threadIdx.x;
+  if (i < n) p[i] = 0;
+}
+
+// Second pass of the fixed split: merge the partials of one (sequence, query
+// head).  grid = (B, Hq), block = head_dim lanes, one per output dim.  The
+// partials of sequence b are slots b*max_chunks .. + ceil(ctx/chunk).  A
+// sequence with one partial was written by the split kernel itself; an empty
+// one gives zeros.
 __global__ __launch_bounds__(kMaxHeadDim) void paged_decode_combine_kernel(
     const float* __restrict__ part_o, const float* __restrict__ part_ml,
-    const int32_t* __restrict__ context_lens, const int32_t* __restrict__ prefix,
-    uint16_t* __restrict__ out, int num_heads, int chunk, int max_chunks, int max_positions,
-    int batch, int num_wgs, int min_steps, float scale_log2e, bool f16) {
+    const int32_t* __restrict__ context_lens, uint16_t* __restrict__ out, int num_heads, int chunk,
+    int max_chunks, int max_positions, float scale_log2e, bool f16) {
   const int b = blockIdx.x, h = blockIdx.y, d = threadIdx.x;
   const int head_dim = blockDim.x;
-  int nparts;
-  int64_t first;
-  if (prefix == nullptr) {
-    const int ctx = min(context_lens[b], max_positions);
-    nparts = ctx <= 0 ? 0 : (ctx + chunk - 1) / chunk;
-    first = (int64_t)b * max_chunks;
-  } else {
-    const int before = prefix[b], nb = prefix[b + 1] - before, total = prefix[batch];
-    const int run = max((total + num_wgs - 1) / num_wgs, min_steps);
-    const int g_first = before / run;
-    nparts = nb <= 0 ? 0 : (before + nb - 1) / run - g_first + 1;
-    first = (int64_t)g_first + b;
-  }
+  const int ctx = min(context_lens[b], max_positions);
+  const int nparts = ctx <= 0 ? 0 : (ctx + chunk - 1) / chunk;
+  const int64_t first = (int64_t)b * max_chunks;
   if (nparts == 1) return;  // written by the split kernel itself
   uint16_t* o = out + ((int64_t)b * num_heads + h) * head_dim + d;
   if (nparts == 0) {  // empty sequence: 0 / (0 + 1e-9)
@@ -1028,64 +1380,87 @@ int virtual_heads_per_cache_head(int group) {
   return rep;
 }
 
-// Whole-sequence mode: KV heads per 8-wave workgroup.  As many as still give
-// one workgroup per CU (256), so that the split inside a workgroup is no finer
-// than needed; it must divide the number of KV heads.
-int whole_sequence_heads_per_workgroup(int64_t batch, int num_kv_heads) {
+// Compute units of the current device (256 on an MI355X), looked up once per
+// device; 256 when no device can be asked (argument checks without a GPU).
+int compute_units() {
+  constexpr int kMaxDevicesSeen = 64;
+  static std::atomic<int> cached[kMaxDevicesSeen];
+  int dev = -1;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevicesSeen) {
+    (void)hipGetLastError();   // not an error of any launch
+    return 256;
+  }
+  int n = cached[dev].load(std::memory_order_relaxed);
+  if (n > 0) return n;
+  if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess ||
+      n <= 0) {
+    (void)hipGetLastError();
+    return 256;
+  }
+  cached[dev].store(n, std::memory_order_relaxed);
+  return n;
+}
+
+// KV heads per 8-wave workgroup (whole-sequence and balanced modes): as many as
+// still give one (sequence, head group) row per CU, so that a sequence is split
+// over the waves of a workgroup no finer than needed; it must divide the number
+// of KV heads.
+int heads_per_workgroup(int64_t batch, int num_kv_heads) {
+  const int cus = compute_units();
   int hpw = 8;
-  while (hpw > 1 && (num_kv_heads % hpw != 0 || batch * (num_kv_heads / hpw) < 256)) hpw /= 2;
+  while (hpw > 1 && (num_kv_heads % hpw != 0 || batch * (num_kv_heads / hpw) < cus)) hpw /= 2;
   return hpw;
 }
 
-// Balanced mode launches at most one workgroup per CU of an MI355X, and never
-// gives a workgroup fewer than 4 steps (128 positions): below that the
-// partials cost more than the split gains.
-constexpr int kMaxBalancedWorkgroups = 256;
-constexpr int kMinBalancedSteps = 4;
+// Balanced mode launches at most one workgroup per CU, and never gives a wave
+// fewer than this many 32-position steps.
+constexpr int kMinBalancedSteps = 1;
 
-// Waves per workgroup = KV heads a workgroup covers: the largest of 8, 4, 2, 1
-// that divides the number of KV heads.
+// Waves per workgroup of the fixed split = KV heads a workgroup covers: the
+// largest of 8, 4, 2, 1 that divides the number of KV heads.
 int waves_per_workgroup(int num_kv_heads) {
   return num_kv_heads % 8 == 0 ? 8 : num_kv_heads % 4 == 0 ? 4 : num_kv_heads % 2 == 0 ? 2 : 1;
 }
 
-// Runs (grid.x) of the balanced split.  grid.y = num_kv_heads / waves per
-// workgroup head groups walk the same runs, so the cap of one workgroup per CU
-// applies to their product.
-int balanced_workgroups(int64_t batch, int64_t max_blocks, int64_t block_size, int num_kv_heads) {
-  const int head_groups = num_kv_heads / waves_per_workgroup(num_kv_heads);
-  const int64_t cap = kMaxBalancedWorkgroups / head_groups > 0
-                          ? kMaxBalancedWorkgroups / head_groups : 1;
-  const int64_t max_steps = batch * ((max_blocks * block_size + kStep - 1) / kStep);
-  const int64_t wgs = (max_steps + kMinBalancedSteps - 1) / kMinBalancedSteps;
-  return (int)(wgs < 1 ? 1 : wgs > cap ? cap : wgs);
-}
-
-// Workspace layout.  Fixed chunks: slots = batch * max_chunks.  Balanced:
-// slots = workgroups + batch, followed by the int32 prefix array [batch + 1].
+// Workspace layout.  Fixed chunks: partials of batch * max_chunks slots, every
+// slot holding all query heads.  Balanced: first the counters, one int32 per
+// (sequence, KV head), padded to 256 bytes; then the partials of slots =
+// sub-runs + rows, a slot holding the query heads of hpw KV heads.
 struct WorkspacePlan {
-  int64_t slots;
+  int64_t records;  // partial records (one query head each)
   int max_chunks;   // fixed-chunk mode only
-  int num_wgs;      // balanced mode only
+  int num_wgs, hpw; // balanced mode only
+  size_t counter_bytes;
   size_t bytes;
 };
 
 bool plan_workspace(int64_t batch, int64_t num_heads, int64_t head_dim, int64_t max_blocks,
                     int64_t block_size, int num_kv_heads, int chunk, WorkspacePlan* plan) {
   if (chunk == 0) {
-    plan->num_wgs = balanced_workgroups(batch, max_blocks, block_size, num_kv_heads);
+    const int hpw = heads_per_workgroup(batch, num_kv_heads);
+    const int parts = 8 / hpw;
+    const int64_t rows_per_seq = num_kv_heads / hpw;
+    const int64_t axis = rows_per_seq * batch * ((max_blocks * block_size + kStep - 1) / kStep);
+    if (axis > INT32_MAX / 2) return false;
+    int64_t wgs = (axis + (int64_t)parts * kMinBalancedSteps - 1) / (parts * kMinBalancedSteps);
+    const int64_t cus = compute_units();
+    wgs = wgs < 1 ? 1 : wgs > cus ? cus : wgs;
+    plan->num_wgs = (int)wgs;
+    plan->hpw = hpw;
     plan->max_chunks = 0;
-    plan->slots = plan->num_wgs + batch;
-    const size_t floats = (size_t)plan->slots * num_heads * (head_dim + 2);
-    plan->bytes = floats * sizeof(float) + (size_t)(batch + 1) * sizeof(int32_t);
-    return batch * ((max_blocks * block_size + kStep - 1) / kStep) <= INT32_MAX;
+    const int64_t slots = wgs * parts + batch * rows_per_seq;
+    plan->records = slots * hpw * (num_heads / num_kv_heads);
+    plan->counter_bytes = ((size_t)batch * num_kv_heads * sizeof(int32_t) + 255) / 256 * 256;
+    plan->bytes = plan->counter_bytes + (size_t)plan->records * (head_dim + 2) * sizeof(float);
+    return true;
   }
   const int64_t mc = (max_blocks * block_size + chunk - 1) / chunk;
   if (batch * mc > INT32_MAX) return false;
-  plan->num_wgs = 0;
+  plan->num_wgs = plan->hpw = 0;
   plan->max_chunks = (int)mc;
-  plan->slots = batch * mc;
-  plan->bytes = (size_t)plan->slots * num_heads * (head_dim + 2) * sizeof(float);
+  plan->records = batch * mc * num_heads;
+  plan->counter_bytes = 0;
+  plan->bytes = (size_t)plan->records * (head_dim + 2) * sizeof(float);
   return true;
 }
 
@@ -1111,7 +1486,7 @@ extern "C" int32_t nvj_paged_decode_whole_sequence_workgroups(int32_t batch, int
   const int64_t heads =
       (int64_t)num_kv_heads * virtual_heads_per_cache_head(num_heads / num_kv_heads);
   if (batch * heads > INT32_MAX) return 0;
-  return batch * ((int)heads / whole_sequence_heads_per_workgroup(batch, (int)heads));
+  return batch * ((int)heads / heads_per_workgroup(batch, (int)heads));
 }
 
 extern "C" size_t nvj_paged_decode_workspace_bytes(int32_t batch, int32_t num_heads,
@@ -1131,15 +1506,16 @@ extern "C" size_t nvj_paged_decode_workspace_bytes(int32_t batch, int32_t num_he
   return plan.bytes;
 }
 
-extern "C" int nvj_paged_decode_launch_phases(void* stream, const void* q, const void* k_cache,
-                                              const void* v_cache, const int32_t* block_tables,
-                                              const int32_t* context_lens, void* out,
-                                              void* workspace, size_t workspace_bytes,
-                                              int32_t batch, int32_t num_heads,
-                                              int32_t num_kv_heads, int32_t head_dim,
-                                              int32_t block_size, int32_t max_blocks,
-                                              int32_t num_blocks, float scale, int32_t chunk,
-                                              int32_t dtype, uint32_t phases) {
+namespace {
+// The launch behind every decode entry point.  `ext_counters` != NULL: the
+// counters of the balanced split live there and `workspace` holds the partials
+// only (no counter header in front of them).
+int launch_decode(void* stream, const void* q, const void* k_cache, const void* v_cache,
+                  const int32_t* block_tables, const int32_t* context_lens, void* out,
+                  void* workspace, size_t workspace_bytes, int32_t* ext_counters, int32_t batch,
+                  int32_t num_heads, int32_t num_kv_heads, int32_t head_dim, int32_t block_size,
+                  int32_t max_blocks, int32_t num_blocks, float scale, int32_t chunk,
+                  int32_t dtype, uint32_t phases) {
   if (dtype != NVJ_DTYPE_BF16 && dtype != NVJ_DTYPE_F16) return NVJ_ERR_BAD_DTYPE;
   const bool f16 = dtype == NVJ_DTYPE_F16;
   const bool whole = chunk == NVJ_CHUNK_WHOLE_SEQUENCE;
@@ -1163,7 +1539,7 @@ extern "C" int nvj_paged_decode_launch_phases(void* stream, const void* q, const
   if ((reinterpret_cast<uintptr_t>(q) | reinterpret_cast<uintptr_t>(k_cache) |
        reinterpret_cast<uintptr_t>(v_cache) | reinterpret_cast<uintptr_t>(out) |
        (whole ? 0 : reinterpret_cast<uintptr_t>(workspace))) & 15u)   // unused in whole mode
-    return NVJ_ERR_WORKSPACE;
+    return NVJ_ERR_ALIGNMENT;
   // the vector-ALU measurement variant exists for one shape family only
   const bool valu = (phases & NVJ_PHASE_VALU_PRODUCTS) != 0;
   if (valu && (head_dim != 128 || f16 || kv_rep != 1 || (group != 4 && group != 8) ||
@@ -1193,7 +1569,7 @@ extern "C" int nvj_paged_decode_launch_phases(void* stream, const void* q, const
   if (whole && max_blocks > 0) {
     if ((int64_t)batch * num_kv_heads > INT32_MAX) return NVJ_ERR_BAD_SHAPE;
     if (!(phases & NVJ_PHASE_SPLITK)) return NVJ_OK;   // there is no second pass
-    const int hpw = whole_sequence_heads_per_workgroup(batch, num_kv_heads);
+    const int hpw = heads_per_workgroup(batch, num_kv_heads);
     const dim3 grid((unsigned)(batch * (num_kv_heads / hpw)));
     if (valu && group == 4) paged_decode_whole_kernel<8, 128, false, 4><<<grid, dim3(512), 0, s>>>(a, hpw);
     else if (valu) paged_decode_whole_kernel<8, 128, false, 8><<<grid, dim3(512), 0, s>>>(a, hpw);
@@ -1204,72 +1580,98 @@ extern "C" int nvj_paged_decode_launch_phases(void* stream, const void* q, const
     return hipGetLastError() == hipSuccess ? NVJ_OK : NVJ_ERR_LAUNCH;
   }
 
-  WorkspacePlan plan = {0, 1, 0, 0};
-  int32_t* prefix = nullptr;
+  WorkspacePlan plan = {0, 1, 0, 0, 0, 0};
   if (max_blocks > 0) {
     if (!plan_workspace(batch, num_heads, head_dim, max_blocks, block_size, num_kv_heads, chunk,
                         &plan))
       return NVJ_ERR_BAD_SHAPE;
-    if (!workspace || workspace_bytes < plan.bytes) return NVJ_ERR_WORKSPACE;
-    a.part_o = static_cast<float*>(workspace);
-    a.part_ml = a.part_o + plan.slots * num_heads * head_dim;
-    if (chunk == 0) prefix = reinterpret_cast<int32_t*>(a.part_ml + plan.slots * num_heads * 2);
+    const size_t header = ext_counters ? 0 : plan.counter_bytes;
+    if (!workspace || workspace_bytes < plan.bytes - plan.counter_bytes + header)
+      return NVJ_ERR_WORKSPACE;
+    int32_t* counters = ext_counters ? ext_counters : static_cast<int32_t*>(workspace);
+    a.part_o = reinterpret_cast<float*>(static_cast<char*>(workspace) + header);
+    a.part_ml = a.part_o + plan.records * head_dim;
+
+    if (chunk == 0) {
+      // one launch: the workgroup that completes a sequence merges it
+      if (phases & NVJ_PHASE_CLEAR_COUNTERS) {
+        const int n = batch * num_kv_heads;
+        zero_int32_kernel<<<dim3((unsigned)((n + 255) / 256)), dim3(256), 0, s>>>(counters, n);
+        if (hipGetLastError() != hipSuccess) return NVJ_ERR_LAUNCH;
+      }
+      if (!(phases & NVJ_PHASE_SPLITK)) return NVJ_OK;
+      const dim3 grid((unsigned)plan.num_wgs);
+#define NVJ_LAUNCH_BALANCED(DV, F16V, VGV)                                      \
+  paged_decode_balanced_kernel<DV, F16V, VGV><<<grid, dim3(512), 0, s>>>(      \
+      a, batch, plan.num_wgs, kMinBalancedSteps, plan.hpw, counters)
+      if (valu && group == 4) NVJ_LAUNCH_BALANCED(128, false, 4);
+      else if (valu) NVJ_LAUNCH_BALANCED(128, false, 8);
+      else if (head_dim == 128 && !f16) NVJ_LAUNCH_BALANCED(128, false, 0);
+      else if (head_dim == 128) NVJ_LAUNCH_BALANCED(128, true, 0);
+      else if (!f16) NVJ_LAUNCH_BALANCED(64, false, 0);
+      else NVJ_LAUNCH_BALANCED(64, true, 0);
+#undef NVJ_LAUNCH_BALANCED
+      return hipGetLastError() == hipSuccess ? NVJ_OK : NVJ_ERR_LAUNCH;
+    }
 
     if (phases & NVJ_PHASE_SPLITK) {
       const int nw = waves_per_workgroup(num_kv_heads);
-      const unsigned gy = (unsigned)(num_kv_heads / nw);
-      // one instantiation per (waves per workgroup, head_dim)
-#define NVJ_FOR_DTYPE(LAUNCH, NWV, DV) \
-  do {                                \
-    if (f16) LAUNCH(NWV, DV, true);   \
-    else LAUNCH(NWV, DV, false);      \
+      const dim3 grid((unsigned)(batch * plan.max_chunks), (unsigned)(num_kv_heads / nw));
+      // one instantiation per (waves per workgroup, head_dim, element type)
+#define NVJ_LAUNCH_FIXED(NWV, DV)                                                             \
+  do {                                                                                        \
+    if (f16)                                                                                  \
+      paged_decode_splitk_kernel<NWV, DV, true><<<grid, dim3(NWV * 64), 0, s>>>(a, chunk,     \
+                                                                                plan.max_chunks); \
+    else                                                                                      \
+      paged_decode_splitk_kernel<NWV, DV, false><<<grid, dim3(NWV * 64), 0, s>>>(a, chunk,    \
+                                                                                 plan.max_chunks); \
   } while (0)
-#define NVJ_FOR_SHAPE(LAUNCH)                             \
-  switch (nw * 1000 + head_dim) {                         \
-    case 8128: NVJ_FOR_DTYPE(LAUNCH, 8, 128); break;      \
-    case 4128: NVJ_FOR_DTYPE(LAUNCH, 4, 128); break;      \
-    case 2128: NVJ_FOR_DTYPE(LAUNCH, 2, 128); break;      \
-    case 1128: NVJ_FOR_DTYPE(LAUNCH, 1, 128); break;      \
-    case 8064: NVJ_FOR_DTYPE(LAUNCH, 8, 64); break;       \
-    case 4064: NVJ_FOR_DTYPE(LAUNCH, 4, 64); break;       \
-    case 2064: NVJ_FOR_DTYPE(LAUNCH, 2, 64); break;       \
-    default: NVJ_FOR_DTYPE(LAUNCH, 1, 64); break;         \
-  }
-      if (chunk == 0) {
-        const dim3 grid((unsigned)plan.num_wgs, gy);
-#define NVJ_LAUNCH_BALANCED(NWV, DV, F16V)                                      \
-  paged_decode_balanced_kernel<NWV, DV, F16V><<<grid, dim3(NWV * 64), 0, s>>>( \
-      a, batch, plan.num_wgs, kMinBalancedSteps, prefix)
-        if (valu && group == 4)
-          paged_decode_balanced_kernel<8, 128, false, 4><<<grid, dim3(512), 0, s>>>(
-              a, batch, plan.num_wgs, kMinBalancedSteps, prefix);
-        else if (valu)
-          paged_decode_balanced_kernel<8, 128, false, 8><<<grid, dim3(512), 0, s>>>(
-              a, batch, plan.num_wgs, kMinBalancedSteps, prefix);
-        else
-          NVJ_FOR_SHAPE(NVJ_LAUNCH_BALANCED)
-#undef NVJ_LAUNCH_BALANCED
-      } else {
-        const dim3 grid((unsigned)(batch * plan.max_chunks), gy);
-#define NVJ_LAUNCH_FIXED(NWV, DV, F16V)                                                    \
-  paged_decode_splitk_kernel<NWV, DV, F16V><<<grid, dim3(NWV * 64), 0, s>>>(a, chunk, \
-                                                                             plan.max_chunks)
-        NVJ_FOR_SHAPE(NVJ_LAUNCH_FIXED)
-#undef NVJ_LAUNCH_FIXED
+      switch (nw * 1000 + head_dim) {
+        case 8128: NVJ_LAUNCH_FIXED(8, 128); break;
+        case 4128: NVJ_LAUNCH_FIXED(4, 128); break;
+        case 2128: NVJ_LAUNCH_FIXED(2, 128); break;
+        case 1128: NVJ_LAUNCH_FIXED(1, 128); break;
+        case 8064: NVJ_LAUNCH_FIXED(8, 64); break;
+        case 4064: NVJ_LAUNCH_FIXED(4, 64); break;
+        case 2064: NVJ_LAUNCH_FIXED(2, 64); break;
+        default: NVJ_LAUNCH_FIXED(1, 64); break;
       }
-#undef NVJ_FOR_SHAPE
-#undef NVJ_FOR_DTYPE
+#undef NVJ_LAUNCH_FIXED
       if (hipGetLastError() != hipSuccess) return NVJ_ERR_LAUNCH;
     }
   } else {
-    chunk = kStep;  // no pages at all: every sequence is empty, combine writes zeros
+    chunk = kStep;  // no pages at all: every sequence is empty, the second pass writes zeros
   }
   if (!(phases & NVJ_PHASE_COMBINE)) return NVJ_OK;
   paged_decode_combine_kernel<<<dim3((unsigned)batch, (unsigned)num_heads), dim3(head_dim), 0, s>>>(
-      a.part_o, a.part_ml, context_lens, prefix, static_cast<uint16_t*>(out), num_heads, chunk,
-      plan.max_chunks, max_blocks * block_size, batch, plan.num_wgs, kMinBalancedSteps,
-      a.scale_log2e, f16);
+      a.part_o, a.part_ml, context_lens, static_cast<uint16_t*>(out), num_heads, chunk,
+      plan.max_chunks, max_blocks * block_size, a.scale_log2e, f16);
   return hipGetLastError() == hipSuccess ? NVJ_OK : NVJ_ERR_LAUNCH;
+}
+
+}  // namespace
+
+extern "C" int nvj_paged_decode_launch_phases(void* stream, const void* q, const void* k_cache,
+                                              const void* v_cache, const int32_t* block_tables,
+                                              const int32_t* context_lens, void* out,
+                                              void* workspace, size_t workspace_bytes,
+                                              int32_t batch, int32_t num_heads,
+                                              int32_t num_kv_heads, int32_t head_dim,
+                                              int32_t block_size, int32_t max_blocks,
+                                              int32_t num_blocks, float scale, int32_t chunk,
+                                              int32_t dtype, uint32_t phases) {
+  return launch_decode(stream, q, k_cache, v_cache, block_tables, context_lens, out, workspace,
+                       workspace_bytes, nullptr, batch, num_heads, num_kv_heads, head_dim,
+                       block_size, max_blocks, num_blocks, scale, chunk, dtype, phases);
+}
+
+extern "C" size_t nvj_paged_decode_counter_bytes(int32_t batch, int32_t num_heads,
+                                                 int32_t num_kv_heads) {
+  if (batch <= 0 || num_heads <= 0 || num_kv_heads <= 0 || num_heads % num_kv_heads != 0) return 0;
+  const size_t heads =
+      (size_t)num_kv_heads * virtual_heads_per_cache_head(num_heads / num_kv_heads);
+  return ((size_t)batch * heads * sizeof(int32_t) + 255) / 256 * 256;
 }
 
 extern "C" int nvj_paged_decode_launch(void* stream, const void* q, const void* k_cache,
@@ -1284,7 +1686,8 @@ extern "C" int nvj_paged_decode_launch(void* stream, const void* q, const void* 
                                         out, workspace, workspace_bytes, batch, num_heads,
                                         num_kv_heads, head_dim, block_size, max_blocks,
                                         num_blocks, scale, chunk, dtype,
-                                        NVJ_PHASE_SPLITK | NVJ_PHASE_COMBINE);
+                                        NVJ_PHASE_SPLITK | NVJ_PHASE_COMBINE |
+                                            NVJ_PHASE_CLEAR_COUNTERS);
 }
 
 // ---------------------------------------------------------------------------
@@ -1322,21 +1725,30 @@ extern "C" int nvj_paged_decode_static_launch(void* stream, const void* q, const
                                               int32_t num_kv_heads, int32_t head_dim,
                                               int32_t block_size, int32_t max_blocks,
                                               int32_t num_blocks, float scale, int32_t dtype) {
-  void* ws = nullptr;
+  // The array starts with the counters, in a region of fixed size, so that they
+  // are the same words whatever the shape of a call: zero when the library is
+  // loaded, and put back to zero by every launch.  The partials follow.
+  constexpr size_t kCounterRegion = 64u << 10;
+  void* base = nullptr;
   if (batch > 0 && max_blocks > 0) {
     const size_t need = nvj_paged_decode_workspace_bytes(batch, num_heads, head_dim, max_blocks,
                                                          block_size, num_kv_heads, 0);
+    const size_t counters = nvj_paged_decode_counter_bytes(batch, num_heads, num_kv_heads);
     // need == 0: invalid arguments, which the launch below reports by name
-    if (need > NVJ_STATIC_SCRATCH_BYTES) return NVJ_ERR_SCRATCH_LIMIT;
+    if (need > 0 && (counters > kCounterRegion ||
+                     need - counters > NVJ_STATIC_SCRATCH_BYTES - kCounterRegion))
+      return NVJ_ERR_SCRATCH_LIMIT;
     if (need > 0) {
-      const int rc = static_scratch_of_current_device(&ws);
+      const int rc = static_scratch_of_current_device(&base);
       if (rc != NVJ_OK) return rc;
     }
   }
-  return nvj_paged_decode_launch(stream, q, k_cache, v_cache, block_tables, context_lens, out, ws,
-                                 ws ? (size_t)NVJ_STATIC_SCRATCH_BYTES : 0, batch, num_heads,
-                                 num_kv_heads, head_dim, block_size, max_blocks, num_blocks, scale,
-                                 0, dtype);
+  char* partials = base ? static_cast<char*>(base) + kCounterRegion : nullptr;
+  return launch_decode(stream, q, k_cache, v_cache, block_tables, context_lens, out, partials,
+                       base ? (size_t)NVJ_STATIC_SCRATCH_BYTES - kCounterRegion : 0,
+                       static_cast<int32_t*>(base), batch, num_heads, num_kv_heads, head_dim,
+                       block_size, max_blocks, num_blocks, scale, 0, dtype,
+                       NVJ_PHASE_SPLITK | NVJ_PHASE_COMBINE);
 }
 
 extern "C" const char* nvj_error_string(int code) {
@@ -1345,7 +1757,8 @@ extern "C" const char* nvj_error_string(int code) {
     case NVJ_ERR_NULL_POINTER: return "a required pointer is NULL";
     case NVJ_ERR_BAD_SHAPE: return "invalid shape or size argument";
     case NVJ_ERR_UNSUPPORTED: return "unsupported head_dim / group size / block size / chunk";
-    case NVJ_ERR_WORKSPACE: return "workspace missing, too small or misaligned";
+    case NVJ_ERR_WORKSPACE: return "workspace missing or too small";
+    case NVJ_ERR_ALIGNMENT: return "a pointer is not 16-byte aligned";
     case NVJ_ERR_LAUNCH: return "kernel launch failed";
     case NVJ_ERR_BAD_DTYPE: return "unknown element type code";
     case NVJ_ERR_SCRATCH_LIMIT:

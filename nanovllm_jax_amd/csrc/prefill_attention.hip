@@ -571,7 +571,7 @@ extern "C" int nvj_prefill_attention_launch(void* stream, const void* q, const v
   if (!q || !k || !v || !cu_seqlens_q || !cu_seqlens_k || !out) return NVJ_ERR_NULL_POINTER;
   if ((reinterpret_cast<uintptr_t>(q) | reinterpret_cast<uintptr_t>(k) |
        reinterpret_cast<uintptr_t>(v) | reinterpret_cast<uintptr_t>(out)) & 15u)
-    return NVJ_ERR_BAD_SHAPE;
+    return NVJ_ERR_ALIGNMENT;
   PrefillArgs a = {};
   a.q = static_cast<const uint4*>(q);
   a.k = static_cast<const uint4*>(k);
@@ -608,7 +608,7 @@ extern "C" int nvj_paged_prefill_attention_launch(
   if (max_blocks > 0 && !block_tables) return NVJ_ERR_NULL_POINTER;
   if ((reinterpret_cast<uintptr_t>(q) | reinterpret_cast<uintptr_t>(k_cache) |
        reinterpret_cast<uintptr_t>(v_cache) | reinterpret_cast<uintptr_t>(out)) & 15u)
-    return NVJ_ERR_BAD_SHAPE;
+    return NVJ_ERR_ALIGNMENT;
   PrefillArgs a = {};
   a.q = static_cast<const uint4*>(q);
   a.k = static_cast<const uint4*>(k_cache);

@@ -120,7 +120,7 @@ extern "C" int nvj_qk_norm_rope_store_launch(void* stream, const void* qkv, int6
   if ((q_norm_weight == nullptr) != (k_norm_weight == nullptr)) return NVJ_ERR_NULL_POINTER;
   if ((reinterpret_cast<uintptr_t>(qkv) | reinterpret_cast<uintptr_t>(k_cache) |
        reinterpret_cast<uintptr_t>(v_cache) | reinterpret_cast<uintptr_t>(q_out)) & 3u)
-    return NVJ_ERR_BAD_SHAPE;
+    return NVJ_ERR_ALIGNMENT;
   const int64_t units = (int64_t)num_tokens * heads_total;
   const int64_t blocks = (units + 3) / 4;
   if (blocks > INT32_MAX) return NVJ_ERR_BAD_SHAPE;

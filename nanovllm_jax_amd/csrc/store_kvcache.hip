@@ -92,7 +92,7 @@ extern "C" int nvj_store_kvcache_launch(void* stream, const void* key, const voi
   if (!key || !value || !k_cache || !v_cache || !slot_mapping) return NVJ_ERR_NULL_POINTER;
   if ((reinterpret_cast<uintptr_t>(key) | reinterpret_cast<uintptr_t>(value) |
        reinterpret_cast<uintptr_t>(k_cache) | reinterpret_cast<uintptr_t>(v_cache)) & 15u)
-    return NVJ_ERR_BAD_SHAPE;
+    return NVJ_ERR_ALIGNMENT;
   const int pieces = (int)(row / 8);
   const int64_t total = (int64_t)num_tokens * pieces;
   const int64_t blocks = (total + 255) / 256;

@@ -30,7 +30,7 @@ from .. import _lib
 from ..layers.activation import silu_and_mul
 from ..layers.attention import Attention
 from ..layers.layernorm import rms_norm
-from ..layers.paged_attention import (choose_split, paged_attention,
+from ..layers.paged_attention import (DecodeWorkspace, choose_split, paged_attention,
                                       paged_decode_workspace_bytes)
 from ..layers.prefill_attention import (paged_prefill_attention,
                                         variable_length_attention_prefill)
@@ -266,6 +266,9 @@ class DecodeStepRunner:
                     # they are gathered back from the cache rows just written
                     flat = (-1, c.num_kv_heads, c.head_dim)
                     sl = context.slot_mapping.long()
+                    if bool((sl < 0).any()):    # a skipped row was never stored
+                        raise ValueError("packed prefill through the fused store needs every "
+                                         "prompt row stored: slot_mapping has negative entries")
                     o = variable_length_attention_prefill(
                         q, attn.k_cache.view(flat)[sl], attn.v_cache.view(flat)[sl],
                         context.cu_seqlens_q, context.cu_seqlens_k, scale=attn.scale)
@@ -321,17 +324,26 @@ class DecodeStepRunner:
         """Eager decode step: logits -> greedy token ids [batch] int64."""
         return self.forward(input_ids, positions, context).argmax(dim=-1)
 
+    def _share_workspace(self, batch, max_blocks, decode_split):
+        """One split workspace for all layers (they run one after the other on
+        one stream), large enough for the balanced split and for the split the
+        context asks for; its counters are zero from the start."""
+        c = self.cfg
+        with torch.cuda.device(self.device):
+            need = max(paged_decode_workspace_bytes(batch, c.num_heads, c.head_dim, max_blocks,
+                                                    c.block_size, c.num_kv_heads, chunk)
+                       for chunk in {0, int(decode_split)})
+        ws = DecodeWorkspace(need, self.device)
+        for a in self.attn:
+            a.workspace = ws
+
     def capture(self, input_ids, positions, context):
         """Capture the whole step in one HIP graph over static input buffers;
         returns ``replay() -> token ids`` (the inputs may be updated in place
         between replays)."""
         c = self.cfg
         batch, max_blocks = context.block_tables.shape
-        ws = torch.empty(paged_decode_workspace_bytes(batch, c.num_heads, c.head_dim, max_blocks,
-                                                      c.block_size, c.num_kv_heads, 0),
-                         dtype=torch.uint8, device=self.device)
-        for a in self.attn:
-            a.workspace = ws
+        self._share_workspace(batch, max_blocks, context.decode_split)
         s = torch.cuda.Stream(self.device)
         s.wait_stream(torch.cuda.current_stream(self.device))
         with torch.cuda.stream(s):
@@ -356,11 +368,7 @@ class DecodeStepRunner:
         to the host.  Returns ``replay() -> token ids of that step``."""
         c = self.cfg
         batch, max_blocks = context.block_tables.shape
-        ws = torch.empty(paged_decode_workspace_bytes(batch, c.num_heads, c.head_dim, max_blocks,
-                                                      c.block_size, c.num_kv_heads, 0),
-                         dtype=torch.uint8, device=self.device)
-        for a in self.attn:
-            a.workspace = ws
+        self._share_workspace(batch, max_blocks, context.decode_split)
         # warm every library handle on a side stream; the warm-up step writes
         # the K/V rows of the current step, which the captured step rewrites
         # with the same values, and does not touch the metadata

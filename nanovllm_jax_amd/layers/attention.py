@@ -101,8 +101,8 @@ class Attention:
         self.block_size = block_size
         self.k_cache = None
         self.v_cache = None
-        # optional caller-owned split-K workspace (uint8 device tensor) shared by
-        # the calls of one stream; None = a fresh one per call
+        # optional caller-owned split workspace (a DecodeWorkspace, or a uint8
+        # device tensor) shared by the calls of one stream; None = a fresh one per call
         self.workspace = None
 
     def set_kv_cache(self, k_cache, v_cache):

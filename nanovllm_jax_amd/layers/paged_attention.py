@@ -14,7 +14,7 @@ import torch
 from .. import _lib
 
 __all__ = ["paged_attention", "paged_decode_workspace_bytes", "default_chunk", "WHOLE_SEQUENCE",
-           "choose_split"]
+           "choose_split", "DecodeWorkspace"]
 
 WHOLE_SEQUENCE = _lib.NVJ_CHUNK_WHOLE_SEQUENCE
 
@@ -55,6 +55,33 @@ def paged_decode_workspace_bytes(batch: int, num_heads: int, head_dim: int,
         batch, num_heads, head_dim, max_blocks, block_size, num_kv_heads, chunk))
 
 
+class DecodeWorkspace:
+    """Split workspace kept across the decode calls of ONE stream.
+
+    The balanced split (``chunk=0``) merges the partials of a sequence inside
+    its one launch, by way of counters at the head of the workspace that must be
+    zero when a launch starts and are zero again when it ends.  This buffer is
+    zeroed when it is created, so a call that is handed a ``DecodeWorkspace`` is
+    a single kernel launch; a plain tensor (contents unknown) costs a small
+    clearing launch in front of every call.  Calls that may overlap in time
+    (different streams) need a workspace each."""
+
+    def __init__(self, nbytes: int, device):
+        self.buffer = torch.zeros(max(int(nbytes), 16), dtype=torch.uint8, device=device)
+        # bytes from the start known to be zero: everything at first, afterwards
+        # the counters of the last call (a launch puts exactly those back to zero;
+        # behind them lie its partials)
+        self.zero_prefix = self.buffer.numel()
+
+    @classmethod
+    def for_shape(cls, batch: int, num_heads: int, head_dim: int, max_blocks: int,
+                  block_size: int, num_kv_heads: int, device, chunk: int = 0):
+        with torch.cuda.device(device):   # the size follows the device's CU count
+            need = paged_decode_workspace_bytes(batch, num_heads, head_dim, max_blocks,
+                                                block_size, num_kv_heads, chunk)
+        return cls(need, device)
+
+
 def choose_split(context_lens_host, num_kv_heads: int, num_heads: int | None = None) -> int:
     """``chunk`` for a batch whose lengths the host knows (the reference's filler
     builds ``context_lens`` from Python ints, ``engine/model_runner.py:334-376``):
@@ -75,7 +102,7 @@ def choose_split(context_lens_host, num_kv_heads: int, num_heads: int | None = N
 
 def paged_attention(q, k_cache, v_cache, block_tables, context_lens, scale, block_size,
                     *, chunk: int = 0, out: torch.Tensor | None = None,
-                    workspace: torch.Tensor | None = None,
+                    workspace: "torch.Tensor | DecodeWorkspace | None" = None,
                     phases: int = _lib.NVJ_PHASE_SPLITK | _lib.NVJ_PHASE_COMBINE) -> torch.Tensor:
     """Decode attention over a block-paged KV cache.
 
@@ -88,13 +115,14 @@ def paged_attention(q, k_cache, v_cache, block_tables, context_lens, scale, bloc
     block_size   positions per page; must equal ``k_cache.shape[1]``
 
     Returns [batch, num_heads, head_dim] in q's dtype.  ``chunk`` (0 = balanced split
-    derived from ``context_lens`` on the device; > 0 = that many positions per
-    workgroup, multiple of 32; ``WHOLE_SEQUENCE`` = each sequence finished inside
-    one workgroup, no workspace and no combine launch, for batches of similar
-    lengths), ``out`` and ``workspace``
-    (uint8 tensor of at least ``paged_decode_workspace_bytes`` bytes) are
-    optional tuning/reuse knobs the reference does not have; ``phases`` selects
-    the split-K launch, the combine launch or both (timing aid).
+    derived from ``context_lens`` on the device, one launch; > 0 = that many
+    positions per workgroup, multiple of 32, plus a combine launch;
+    ``WHOLE_SEQUENCE`` = each sequence finished inside one workgroup, no workspace,
+    for batches of similar lengths), ``out`` and ``workspace`` (a
+    ``DecodeWorkspace``, or a uint8 tensor of at least
+    ``paged_decode_workspace_bytes`` bytes whose counters are then cleared by an
+    extra small launch) are optional tuning/reuse knobs the reference does not
+    have; ``phases`` selects the launches (timing aid).
     """
     lib = _lib.load()
     _check_device_tensor(q, "q", None, 3)
@@ -123,6 +151,18 @@ def paged_attention(q, k_cache, v_cache, block_tables, context_lens, scale, bloc
         _require(out.shape == q.shape and out.device == dev, "out must match q")
     need = int(lib.nvj_paged_decode_workspace_bytes(batch, num_heads, head_dim, max_blocks,
                                                     bs, num_kv_heads, chunk)) if batch and max_blocks else 0
+    if isinstance(workspace, DecodeWorkspace):
+        # its counters are zero between calls, unless a call of a smaller shape
+        # has since written partials where this call's counters lie
+        counters = int(lib.nvj_paged_decode_counter_bytes(batch, num_heads, num_kv_heads)) \
+            if chunk == 0 and batch and max_blocks else 0
+        if counters > workspace.zero_prefix:
+            phases = int(phases) | _lib.NVJ_PHASE_CLEAR_COUNTERS
+        if chunk >= 0 and batch and max_blocks:
+            workspace.zero_prefix = counters
+        workspace = workspace.buffer
+    else:
+        phases = int(phases) | _lib.NVJ_PHASE_CLEAR_COUNTERS
     if workspace is None:
         workspace = torch.empty(max(need, 16), dtype=torch.uint8, device=dev)
     else:

@@ -28,7 +28,7 @@ def test_library_exports_every_declared_symbol():
     lib = _lib.load()
     assert lib.nvj_abi_version() == _lib.NVJ_ABI_VERSION
     assert lib.nvj_error_string(0) == b"ok"
-    for code in range(-7, 0):
+    for code in range(-8, 0):
         assert lib.nvj_error_string(code) not in (b"ok", b"unknown error code")
 
 
@@ -55,7 +55,7 @@ def test_argument_validation_without_a_gpu():
     assert call(dtype=3) == -6
     assert call(batch=0) == 0              # empty batch: nothing to do
     assert call(ptr=0) == -1
-    assert call(ptr=0x1004) == -4          # misaligned
+    assert call(ptr=0x1004) == -8          # misaligned
     assert L(None, 0x1000, 0x1000, 0x1000, 0x1000, 0x1000, 0x1000, 0x1000, 16, 2, 32, 8, 128, 256,
              4, 16, 0.1, 0, 0) == -4       # workspace too small
     # the vector-ALU measurement variant exists for group 4 or 8, head_dim 128, bf16 only
@@ -89,11 +89,13 @@ def test_workspace_and_chunk_queries():
     need = paged_decode_workspace_bytes(64, 32, 128, 16, 256, 8, 256)
     assert need == 64 * 16 * 32 * (128 + 2) * 4
     assert paged_decode_workspace_bytes(64, 32, 128, 16, 256, 8, 100) == 0   # bad chunk
-    # balanced split: one partial slot per workgroup (<= 256) plus one per sequence,
-    # then batch + 1 prefix sums
+    # balanced split (no GPU here: 256 compute units assumed): counters, one int32 per
+    # (sequence, KV head) padded to 256 bytes, then one partial slot per wave part of a
+    # workgroup (<= 256 workgroups) plus one per (sequence, head group) row; at batch 64
+    # a workgroup is 2 KV heads x 4 parts, at batch 2 it is 1 KV head x 8 parts
     assert paged_decode_workspace_bytes(64, 32, 128, 16, 256, 8, 0) == \
-        (256 + 64) * 32 * (128 + 2) * 4 + 65 * 4
-    assert paged_decode_workspace_bytes(2, 8, 128, 1, 32, 8, 0) == (1 + 2) * 8 * 130 * 4 + 3 * 4
+        2048 + (256 * 4 + 64 * 4) * 2 * 4 * (128 + 2) * 4
+    assert paged_decode_workspace_bytes(2, 8, 128, 1, 32, 8, 0) == 256 + (2 * 8 + 2 * 8) * 130 * 4
 
 
 def test_host_mirror_refuses_cpu_tensors():

@@ -157,6 +157,131 @@ def test_balanced_split_many_ragged_sequences(B, seed):
     assert_close_bf16(fixed, want, what=f"fixed chunk B={B}")
 
 
+@pytest.mark.parametrize("B,Hq,Hkv,D,lo,hi", [
+    (3, 32, 8, 128, 0, 3000),      # 1 KV head x 8 parts per workgroup, rows over many workgroups
+    (64, 32, 8, 128, 0, 900),      # 2 x 4, runs cross rows of different head groups
+    (64, 16, 8, 128, 500, 512),    # 2 x 4, every row exactly one workgroup (no partials)
+    (130, 16, 8, 128, 0, 400),     # 4 x 2
+    (140, 8, 4, 64, 0, 300),       # head_dim 64, 2 x 4
+    (90, 12, 6, 128, 0, 500),      # 6 KV heads: 2 per workgroup
+    (40, 5, 5, 128, 0, 700),       # 5 KV heads: 1 per workgroup
+    (300, 8, 8, 128, 0, 200)])     # 8 x 1
+def test_balanced_split_every_workgroup_shape(B, Hq, Hkv, D, lo, hi):
+    """chunk = 0 picks the KV heads per workgroup from the batch and head counts; every
+    shape, with rows that are finished inside one workgroup, rows shared by parts of a
+    workgroup (merged in LDS) and rows shared by workgroups (merged by the wave that
+    completes them), against the oracle."""
+    print(f"case balanced shapes B={B} Hq={Hq} Hkv={Hkv} D={D}", flush=True)
+    rng = np.random.Generator(np.random.PCG64(B * 7 + Hkv))
+    bs = 64
+    ctx = rng.integers(lo, hi + 1, size=B)
+    if lo == 0:
+        ctx[rng.integers(0, B, size=max(1, B // 9))] = 0
+        ctx[rng.integers(0, B)] = hi * 3            # one long sequence
+    NB = int((-(-ctx // bs)).sum()) + 2
+    q, kc, vc, bt, ctx = make_problem(900 + B, B, Hq, Hkv, D, bs, NB, ctx)
+    scale = 1.0 / np.sqrt(D)
+    got = run_hip(q, kc, vc, bt, ctx, scale, bs, 0)
+    want = oracle(q, kc, vc, bt, ctx, scale, bs)
+    assert_close_bf16(got, want, what=f"balanced shapes B={B} Hkv={Hkv}")
+    assert not got[ctx == 0].any()
+
+
+@pytest.mark.parametrize("B,Hkv", [(6, 8), (64, 8), (300, 4)])
+def test_balanced_split_is_one_launch_that_leaves_its_counters_zero(B, Hkv):
+    """With a DecodeWorkspace (counters zero from the start) a chunk = 0 call is a single
+    kernel that merges shared rows itself and puts every counter back to zero: 20 replays
+    of one captured launch, the lengths changing before every replay (growing, shrinking,
+    emptied, so the rows that are shared and the waves that merge them change too), each
+    equal to an eager call on a fresh workspace and within the bar of the oracle."""
+    print(f"case balanced one launch, 20 replays B={B} Hkv={Hkv}", flush=True)
+    import torch
+    from nanovllm_jax_amd import _lib, paged_attention
+    from nanovllm_jax_amd.layers.paged_attention import DecodeWorkspace
+    Hq, D, bs = 2 * Hkv, 128, 64
+    rng = np.random.Generator(np.random.PCG64(31 + B))
+    cap = rng.integers(64, 1500, size=B)               # positions each sequence owns pages for
+    q, kc, vc, bt, cap = make_problem(77 + B, B, Hq, Hkv, D, bs,
+                                      int((-(-cap // bs)).sum()) + 1, cap)
+    dev = "cuda:0"
+    qt, kt, vt = bits_to_torch(q, dev), bits_to_torch(kc, dev), bits_to_torch(vc, dev)
+    btt, ct = torch.from_numpy(bt).to(dev), torch.from_numpy(cap).to(dev)
+    out = torch.empty_like(qt)
+    ws = DecodeWorkspace.for_shape(B, Hq, D, bt.shape[1], bs, Hkv, dev)
+    counter_bytes = -(-B * Hkv * 4 // 256) * 256
+    call = lambda: paged_attention(qt, kt, vt, btt, ct, 0.088, bs, chunk=0, out=out,
+                                   workspace=ws, phases=_lib.NVJ_PHASE_SPLITK)
+    s = torch.cuda.Stream(dev)
+    s.wait_stream(torch.cuda.current_stream(dev))
+    with torch.cuda.stream(s):
+        call()
+    torch.cuda.current_stream(dev).wait_stream(s)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        call()
+    for step in range(20):
+        new_ctx = (cap * rng.random(B)).astype(np.int32)
+        new_ctx[rng.integers(0, B, size=2)] = 0
+        if step % 5 == 0:
+            new_ctx = cap.copy()
+        ct.copy_(torch.from_numpy(new_ctx).to(dev))
+        out.fill_(7.0)
+        graph.replay()
+        torch.cuda.synchronize()
+        replayed = torch_to_bits(out).copy()
+        assert not ws.buffer[:counter_bytes].any(), f"replay {step} left a counter set"
+        eager = paged_attention(qt, kt, vt, btt, ct, 0.088, bs, chunk=0)   # fresh workspace
+        torch.cuda.synchronize()
+        assert np.array_equal(replayed, torch_to_bits(eager)), f"replay {step} differs from eager"
+        want = oracle(q, kc, vc, bt, new_ctx, 0.088, bs)
+        assert_close_bf16(replayed, want, what=f"one-launch replay {step}")
+
+
+def test_decode_workspace_reused_across_shapes():
+    """One DecodeWorkspace serving calls of different shapes: the counters of a larger
+    batch lie where a smaller batch left partials, which the binding knows and clears."""
+    print("case DecodeWorkspace across shapes", flush=True)
+    import torch
+    from nanovllm_jax_amd import paged_attention
+    from nanovllm_jax_amd.layers.paged_attention import DecodeWorkspace
+    dev, D, bs = "cuda:0", 128, 64
+    ws = DecodeWorkspace(32 << 20, dev)
+    for seed, B, Hq, Hkv, chunk in [(1, 3, 32, 8, 0), (2, 90, 16, 8, 0), (3, 5, 16, 8, 64),
+                                    (4, 200, 8, 8, 0), (5, 2, 8, 2, 0)]:
+        rng = np.random.Generator(np.random.PCG64(seed))
+        ctx = rng.integers(0, 1200, size=B)
+        q, kc, vc, bt, ctx = make_problem(seed, B, Hq, Hkv, D, bs,
+                                          int((-(-ctx // bs)).sum()) + 1, ctx)
+        out = paged_attention(bits_to_torch(q, dev), bits_to_torch(kc, dev),
+                              bits_to_torch(vc, dev), torch.from_numpy(bt).to(dev),
+                              torch.from_numpy(ctx).to(dev), 0.088, bs, chunk=chunk, workspace=ws)
+        torch.cuda.synchronize()
+        assert_close_bf16(torch_to_bits(out), oracle(q, kc, vc, bt, ctx, 0.088, bs),
+                          what=f"shared workspace, call {seed}")
+
+
+def test_balanced_split_plain_entry_point_clears_dirty_counters():
+    """nvj_paged_decode_launch promises that the workspace need not be initialised: it
+    clears the counters itself.  Fill the workspace with ones and call it."""
+    print("case balanced, dirty workspace", flush=True)
+    import torch
+    from nanovllm_jax_amd import paged_attention
+    from nanovllm_jax_amd.layers.paged_attention import paged_decode_workspace_bytes
+    B, Hq, Hkv, D, bs, NB = 10, 32, 8, 128, 64, 200
+    ctx = [1000, 5, 0, 640, 77, 1200, 64, 333, 2, 900]
+    q, kc, vc, bt, ctx = make_problem(91, B, Hq, Hkv, D, bs, NB, ctx)
+    dev = "cuda:0"
+    ws = torch.full((paged_decode_workspace_bytes(B, Hq, D, bt.shape[1], bs, Hkv, 0),), 0xFF,
+                    dtype=torch.uint8, device=dev)
+    out = paged_attention(bits_to_torch(q, dev), bits_to_torch(kc, dev), bits_to_torch(vc, dev),
+                          torch.from_numpy(bt).to(dev), torch.from_numpy(ctx).to(dev), 0.088, bs,
+                          chunk=0, workspace=ws)
+    torch.cuda.synchronize()
+    assert_close_bf16(torch_to_bits(out), oracle(q, kc, vc, bt, ctx, 0.088, bs),
+                      what="dirty workspace")
+
+
 def test_balanced_split_all_empty_and_single_position():
     print("case balanced all-empty / single position", flush=True)
     B, Hq, Hkv, D, bs, NB = 9, 32, 8, 128, 256, 12
@@ -292,7 +417,8 @@ def test_whole_sequence_mode_needs_no_workspace_and_ignores_garbage():
 def test_decode_call_replays_in_a_hip_graph(chunk):
     """The decode launch(es) captured once and replayed with the lengths and the
     query updated in place between replays give what eager calls give, every
-    time (balanced split + combine, and the one-launch whole-sequence split)."""
+    time (balanced split behind its counter-clearing launch, and the whole-sequence
+    split)."""
     print(f"case decode graph replays chunk={chunk}", flush=True)
     import torch
     from nanovllm_jax_amd import paged_attention

@@ -1,7 +1,7 @@
 """The allocation-free decode entry point (nvj_paged_decode_static_launch, its
 workspace in a device array inside the library) against
 nvj_paged_decode_launch(chunk = 0) with a caller-owned workspace: bit-equal
-outputs on two calls in a row, the second with a smaller input, and within the
+outputs on calls in a row, the second with a smaller input, and within the
 attention parity bar of the CPU oracle.  Both are called through the C ABI."""
 import numpy as np
 import pytest
@@ -48,8 +48,11 @@ def test_static_scratch_entry_point_matches_workspace_entry_point():
     scale = float(1.0 / np.sqrt(D))
     # first call: ragged, several partials per sequence; second call: smaller in
     # every dimension, so most of what the first left in the array is stale
+    # third call: more sequences again, so its counters are words the smaller call did
+    # not use
     cases = [(21, 12, 32, 8, 64, [3000, 17, 0, 1024, 2049, 700, 1, 256, 1500, 333, 2900, 64]),
-             (22, 3, 16, 8, 8, [700, 90, 257])]
+             (22, 3, 16, 8, 8, [700, 90, 257]),
+             (23, 40, 16, 8, 128, [300 + 7 * i for i in range(40)])]
     for seed, B, Hq, Hkv, NB, ctx in cases:
         print(f"case static seed={seed} B={B} Hq={Hq} Hkv={Hkv}", flush=True)
         prob = make_problem(seed, B, Hq, Hkv, D, bs, NB, ctx)
