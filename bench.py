@@ -1,16 +1,20 @@
 #!/usr/bin/env python3
 """Benchmark of the paged-decode hot path on one MI355X.
 
-A step is one paged decode attention call (split-K launch + combine launch)
-over one synthetic batch that is already resident in HBM.  The default
-workload is C2 (Qwen3-8B shape: B=64, Hq=32, Hkv=8, D=128, page 256,
-ctx 4096).  One JSON line is printed on stdout.
+A step is one paged decode attention call over one synthetic batch that is
+already resident in HBM.  The default workload is C2 (Qwen3-8B shape: B=64,
+Hq=32, Hkv=8, D=128, page 256, ctx 4096) in the balanced split (chunk 0, the
+mode a caller that does not know the lengths on the host gets), which is one
+kernel launch.  One JSON line is printed on stdout.
 
   value                GB/s = algorithmic bytes per call / mean time per call
-  roofline.achieved    same bytes / mean duration of the split-K kernel alone,
+  roofline.achieved    same bytes / mean duration of the attention kernel alone,
                        timed with events on the launch stream
-  cpu_baseline         the CPU oracle (a NumPy port of the reference's pure-JAX
-                       paged attention) on a bounded sample of the same batch
+  cpu_baseline         the CPU oracle on a bounded sample of the same batch: the
+                       C restatement (OpenMP), and under "literal" the NumPy
+                       restatement of the reference's own materialising algorithm
+  others               the other workloads and neighbours of the path, each
+                       timed in this same run (skipped with --no-others)
 """
 from __future__ import annotations
 
@@ -28,12 +32,14 @@ if ROOT not in sys.path:
 
 HBM_PEAK_GBPS = 8000.0
 
-# HBM bytes per decode launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of
-# this very command, scaled by the same counters over a plain 1 GiB copy
-# (FETCH_SIZE x1.9999, WRITE_SIZE x1.0).  Keyed by (workload, chunk); other
-# configurations report null.
-MEASURED_TRAFFIC_BYTES = {("C2", 0): 1_080_210_000, ("C2", 1024): 1_080_188_000,
-                          ("C2", -1): 1_074_909_000}
+# HBM bytes per decode launch as measured by rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
+# runs of this command on an earlier day, scaled by the same counters over a plain
+# 1 GiB copy.  Not measured by the run that prints them: reported with the file
+# they come from, and only for the exact configuration that was profiled.
+PROFILED_TRAFFIC = {
+    ("C2", 0, "bf16", "mfma"): (None, "profiles/paged_decode_balanced_kernel_C2.md"),
+    ("C2", -1, "bf16", "mfma"): (1_074_909_000, "profiles/paged_decode_whole_kernel_C2.md"),
+}
 
 
 def device_inputs(w, torch, dev, dt=None):
@@ -141,13 +147,50 @@ def cpu_baseline(w, q, kc, vc, budget_s=20.0, dtype="bf16"):
     byts = algorithmic_bytes(w.context_lens[:n], n, w.num_heads, w.num_kv_heads, w.head_dim,
                              w.max_blocks)
     pos = int(w.context_lens[:n].sum())
-    return {"value": round(byts / med / 1e9, 3), "unit": "GB/s", "cores": cores, "kind": "port",
-            "us_per_call_full_batch": round(med / max(pos, 1) * int(w.context_lens.sum()) * 1e6, 1),
-            "sample": f"{impl}, {cores} threads, first {n} of {w.batch} sequences of {w.name} "
-                      f"({pos} positions), median of {len(times)} calls of {med * 1e3:.1f} ms"}
+    rec = {"value": round(byts / med / 1e9, 3), "unit": "GB/s", "cores": cores, "kind": "port",
+           "us_per_call_full_batch": round(med / max(pos, 1) * int(w.context_lens.sum()) * 1e6, 1),
+           "sample": f"{impl}, {cores} threads, first {n} of {w.batch} sequences of {w.name} "
+                     f"({pos} positions), median of {len(times)} calls of {med * 1e3:.1f} ms; "
+                     "a streaming restatement written for speed, which flatters the CPU: the "
+                     "reference's own algorithm is under 'literal'"}
+    if dtype == "bf16":
+        rec["literal"] = cpu_baseline_literal(w, qb, kb, vb, budget_s / 2)
+    return rec
 
 
-def bench_decode_step(args, torch):
+def cpu_baseline_literal(w, qb, kb, vb, budget_s):
+    """The reference's algorithm as it stands (layers/pallas_attention.py:188-236:
+    gather the pages of the whole table, repeat K/V for the query group, convert to
+    fp32, masked softmax over every table position), restated in NumPy, on the
+    first sequences of the batch: as many as keep one call within the budget and
+    the fp32 copies within a few GiB."""
+    from nanovllm_jax_amd.workloads import algorithmic_bytes
+    from oracle.paged_attention_oracle import paged_decode_attention_vectorized_ref
+    per_seq = 2 * w.max_blocks * w.block_size * w.num_heads * w.head_dim * 4   # K and V, fp32
+    n_max = max(1, min(w.batch, (8 << 30) // per_seq))
+
+    def call(n):
+        t0 = time.perf_counter()
+        paged_decode_attention_vectorized_ref(qb[:n], kb, vb, w.block_tables[:n],
+                                              w.context_lens[:n], w.scale, w.block_size)
+        return time.perf_counter() - t0
+
+    n, t = 1, call(1)
+    while n < n_max and t * 2 * 2 < budget_s:       # one more timed call must still fit
+        n = min(n_max, n * 2)
+        t = call(n)
+    t = min(t, call(n)) if t * 2 < budget_s else t
+    byts = algorithmic_bytes(w.context_lens[:n], n, w.num_heads, w.num_kv_heads, w.head_dim,
+                             w.max_blocks)
+    pos = int(w.context_lens[:n].sum())
+    return {"value": round(byts / t / 1e9, 3), "unit": "GB/s", "cores": 1, "kind": "port",
+            "us_per_call_full_batch": round(t / max(pos, 1) * int(w.context_lens.sum()) * 1e6, 1),
+            "sample": f"NumPy restatement of paged_decode_attention_vectorized, first {n} of "
+                      f"{w.batch} sequences of {w.name} ({pos} positions), best of the calls "
+                      f"made, {t * 1e3:.0f} ms"}
+
+
+def decode_step_record(steps, warmup, torch):
     """Whole-model decode step at the Qwen3-0.6B shape: 28 layers, B=128, every
     sequence at context 1024, page 256, random bf16 weights, greedy pick; the
     step is one HIP graph.  Reports decode tokens/s."""
@@ -162,28 +205,28 @@ def bench_decode_step(args, torch):
     eager = runner.step(ids, pos, ctx).clone()
     replay = runner.capture(ids, pos, ctx)
     same = bool(torch.equal(replay(), eager))
-    for _ in range(args.warmup):
+    for _ in range(warmup):
         replay()
-    ms, wall = timed(replay, args.steps, torch)
-    ms_eager, _ = timed(lambda: runner.step(ids, pos, ctx), max(3, args.steps // 10), torch)
+    ms, wall = timed(replay, steps, torch)
+    ms_eager, _ = timed(lambda: runner.step(ids, pos, ctx), max(3, steps // 10), torch)
     kv_bytes = cfg.num_layers * batch * ctx_len * cfg.num_kv_heads * cfg.head_dim * 2 * 2
     rec = {"metric": "decode tokens/s, Qwen3-0.6B shape whole-model decode step", "value":
-           round(batch / (ms * 1e-3), 1), "unit": "tokens/s", "n_gpus": 1, "steps": args.steps,
-           "warmup": args.warmup, "ms_per_step": round(wall, 4), "higher_is_better": True,
+           round(batch / (ms * 1e-3), 1), "unit": "tokens/s", "n_gpus": 1, "steps": steps,
+           "warmup": warmup, "ms_per_step": round(wall, 4), "higher_is_better": True,
            "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
            "config": {"workload": "C5: 28 layers, hidden 1024, Hq=16, Hkv=8, D=128, vocab 151936, "
                                   "B=128, ctx=1024, page=256, random-init weights, greedy",
                       "step": "one HIP graph: embedding .. LM head .. argmax",
                       "kv_bytes_per_step": kv_bytes},
            "ms_per_step_eager": round(ms_eager, 4), "graph_matches_eager": same}
-    print(json.dumps(rec), flush=True)
-    return 0
+    del runner, replay
+    return rec
 
 
 MFMA_BF16_PEAK_TFLOPS = 2500.0
 
 
-def bench_prefill(args, torch):
+def prefill_record(lens, prefix, steps, warmup, torch):
     """Variable-length causal prefill attention at the Qwen3-8B head shape
     (Hq=32, Hkv=8, D=128): 8 prompts of 4096 tokens, packed.  Reports TFLOP/s
     (4 * Hq * D flop per visible (query, key) pair) against the dense bf16 MFMA
@@ -191,8 +234,6 @@ def bench_prefill(args, torch):
     from nanovllm_jax_amd import paged_prefill_attention, variable_length_attention_prefill
     dev = torch.device("cuda:0")
     hq, hkv, d = 32, 8, 128
-    lens = [int(x) for x in args.prefill_lens.split(",")]
-    prefix = int(args.prefill_prefix)
     cu = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
     g = torch.Generator(device=dev)
     g.manual_seed(7)
@@ -221,15 +262,15 @@ def bench_prefill(args, torch):
         cu_k = torch.from_numpy(np.concatenate([[0], np.cumsum(lens_k)]).astype(np.int32)).to(dev)
         bt_t = torch.from_numpy(bt).to(dev)
         fn = lambda: paged_prefill_attention(q, kc, vc, bt_t, cu_t, cu_k, d ** -0.5, out=out)
-    for _ in range(args.warmup):
+    for _ in range(warmup):
         fn()
-    ms, wall = timed(fn, args.steps, torch)
+    ms, wall = timed(fn, steps, torch)
     pairs = sum(n * (n + 1) // 2 + n * prefix for n in lens)
     flops = 4.0 * hq * d * pairs
     tflops = flops / (ms * 1e-3) / 1e12
     rec = {"metric": "prefill attention TFLOP/s (causal, varlen, Qwen3-8B head shape)",
-           "value": round(tflops, 1), "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps,
-           "warmup": args.warmup, "ms_per_step": round(wall, 4), "higher_is_better": True,
+           "value": round(tflops, 1), "unit": "TFLOP/s", "n_gpus": 1, "steps": steps,
+           "warmup": warmup, "ms_per_step": round(wall, 4), "higher_is_better": True,
            "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
            "config": {"workload": f"prefill: Hq={hq} Hkv={hkv} D={d}, prompt lengths {lens}" +
                                   (f" behind {prefix} cached positions each (paged cache)"
@@ -239,8 +280,103 @@ def bench_prefill(args, torch):
                         "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
                         "frac": round(tflops / MFMA_BF16_PEAK_TFLOPS, 4), "traffic": None,
                         "kernel": "prefill_attention_kernel", "kernel_us": round(ms * 1e3, 1)}}
-    print(json.dumps(rec), flush=True)
-    return 0
+    return rec
+
+
+def decode_record(name, chunk, dtype, products, steps, warmup, torch, dev, in_graph=False,
+                  keep_inputs=False):
+    """Time the decode call (and the KV store) on one workload.  Returns the
+    measurements, plus the device inputs when `keep_inputs`."""
+    from nanovllm_jax_amd import _lib, paged_attention, store_kv_to_cache
+    from nanovllm_jax_amd.layers.paged_attention import DecodeWorkspace
+    from nanovllm_jax_amd.workloads import algorithmic_bytes, make_workload
+    w = make_workload(name)
+    dt = torch.float16 if dtype == "f16" else torch.bfloat16
+    q, kc, vc, bt, ctx, slots, k_new, v_new = device_inputs(w, torch, dev, dt)
+    # one workspace kept across the calls of this stream: its counters are zero
+    # between calls, so a balanced call is a single launch
+    ws = DecodeWorkspace.for_shape(w.batch, w.num_heads, w.head_dim, w.max_blocks, w.block_size,
+                                   w.num_kv_heads, dev, chunk)
+    out = torch.empty_like(q)
+    kflat = kc.view(-1, w.num_kv_heads, w.head_dim)
+    vflat = vc.view(-1, w.num_kv_heads, w.head_dim)
+    variant = _lib.NVJ_PHASE_VALU_PRODUCTS if products == "valu" else 0
+
+    def decode(phases=_lib.NVJ_PHASE_SPLITK | _lib.NVJ_PHASE_COMBINE):
+        paged_attention(q, kc, vc, bt, ctx, w.scale, w.block_size, chunk=chunk, out=out,
+                        workspace=ws, phases=phases | variant)
+
+    def store():
+        store_kv_to_cache(k_new, v_new, kflat, vflat, slots)
+
+    store()
+    for _ in range(warmup):
+        decode()
+    ms_call, ms_wall = timed(decode, steps, torch)
+    # the attention kernel alone: all there is for chunk 0 and -1, the first of the
+    # two launches for a fixed chunk
+    ms_kernel = ms_call if chunk <= 0 else timed(lambda: decode(_lib.NVJ_PHASE_SPLITK), steps,
+                                                 torch)[0]
+    ms_store, _ = timed(store, steps, torch)
+    m = {"workload": w, "ms_call": ms_call, "ms_wall": ms_wall, "ms_kernel": ms_kernel,
+         "ms_store": ms_store,
+         "bytes": algorithmic_bytes(w.context_lens, w.batch, w.num_heads, w.num_kv_heads,
+                                    w.head_dim, w.max_blocks)}
+    if in_graph:
+        m["ms_graph"] = timed_in_graph(decode, torch)
+        m["ms_store_graph"] = timed_in_graph(store, torch)
+    if keep_inputs:
+        m["inputs"] = (q, kc, vc)
+    return m
+
+
+def brief(m):
+    """One workload's line in the `others` block."""
+    gbps = m["bytes"] / (m["ms_call"] * 1e-3) / 1e9
+    r = {"us_per_call": round(m["ms_call"] * 1e3, 2), "GB/s": round(gbps, 1),
+         "pct_of_hbm_peak": round(100.0 * gbps / HBM_PEAK_GBPS, 2)}
+    if "ms_graph" in m:
+        r["us_per_call_in_graph"] = round(m["ms_graph"] * 1e3, 2)
+        r["store_us_per_call_in_graph"] = round(m["ms_store_graph"] * 1e3, 2)
+    return r
+
+
+def others_block(args, torch, dev):
+    """The numbers quoted beside the headline, measured in this same run: the
+    other split of C2, the other workloads in the default split, C1 inside a HIP
+    graph (it is launch-bound), the prefill kernel and the whole-model decode
+    step.  Fewer timed steps than the headline; every figure says what it is."""
+    st, wu = max(10, args.steps // 2), max(5, args.warmup)
+    o = {"split": "balanced (chunk 0, one launch) unless a key says otherwise", "steps": st}
+
+    def run(key, fn):
+        try:
+            o[key] = fn()
+        except Exception as e:          # one failing extra must not take the headline down
+            o[key] = {"error": f"{type(e).__name__}: {e}"}
+
+    run("C2_whole_sequence_split", lambda: brief(decode_record("C2", -1, "bf16", "mfma", st, wu,
+                                                              torch, dev)))
+    run("C1", lambda: brief(decode_record("C1", 0, "bf16", "mfma", st, wu, torch, dev,
+                                          in_graph=True)))
+    run("C5_layer", lambda: brief(decode_record("C5", 0, "bf16", "mfma", st, wu, torch, dev)))
+    run("C4", lambda: brief(decode_record("C4", 0, "bf16", "mfma", st, wu, torch, dev)))
+    run("C3", lambda: brief(decode_record("C3", 0, "bf16", "mfma", st, wu, torch, dev)))
+
+    def prefill():
+        r = prefill_record([4096] * 8, 0, max(5, st // 5), 2, torch)
+        return {"TFLOP/s": r["value"], "pct_of_mfma_bf16_peak": round(100 * r["roofline"]["frac"], 2),
+                "us_per_call": r["roofline"]["kernel_us"], "workload": r["config"]["workload"]}
+    run("prefill_8x4096", prefill)
+
+    def step():
+        r = decode_step_record(max(5, st // 5), 2, torch)
+        return {"tokens/s": r["value"], "ms_per_step": round(128 / r["value"] * 1e3, 4),
+                "ms_per_step_eager": r["ms_per_step_eager"],
+                "graph_matches_eager": r["graph_matches_eager"],
+                "workload": r["config"]["workload"]}
+    run("C5_decode_step", step)
+    return o
 
 
 def main():
@@ -249,18 +385,19 @@ def main():
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--workload", default="C2", choices=["C1", "C2", "C3", "C4", "C5", "R1"])
-    ap.add_argument("--chunk", type=int, default=None,
-                    help="split mode: 0 = balanced, > 0 = positions per workgroup, -1 = whole "
-                         "sequence per workgroup; default: what the host filler would pick from "
-                         "the workload's lengths (layers.paged_attention.choose_split)")
+    ap.add_argument("--chunk", type=int, default=0,
+                    help="split mode: 0 = balanced (one launch, the default), > 0 = positions "
+                         "per workgroup plus a combine launch, -1 = whole sequence per workgroup")
     ap.add_argument("--dtype", default="bf16", choices=["bf16", "f16"],
                     help="cache / q / out dtype; f16 is what the reference's own timing "
                          "scripts use")
     ap.add_argument("--products", default="mfma", choices=["mfma", "valu"],
-                    help="valu: time the measurement variant of the split-K kernel that does "
+                    help="valu: time the measurement variant of the kernel that does "
                          "Q.K and P.V with vector-ALU dot products (group 4 or 8, bf16, "
                          "balanced or whole-sequence split)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-others", action="store_true",
+                    help="skip the `others` block (the other workloads, prefill, decode step)")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run a plain 1 GiB device-to-device copy a few times, so a "
                          "counter run has a kernel of known traffic to scale against")
@@ -287,40 +424,17 @@ def main():
         print("bench.py: no GPU visible; the paged-decode path has no CPU implementation",
               file=sys.stderr)
         return 1
-    from nanovllm_jax_amd import _lib, paged_attention, store_kv_to_cache
-    from nanovllm_jax_amd.layers.paged_attention import DecodeWorkspace, choose_split
-    from nanovllm_jax_amd.workloads import algorithmic_bytes, make_workload
 
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
     if args.decode_step:
-        return bench_decode_step(args, torch)
+        print(json.dumps(decode_step_record(args.steps, args.warmup, torch)), flush=True)
+        return 0
     if args.prefill:
-        return bench_prefill(args, torch)
-    w = make_workload(args.workload)
-    dt = torch.float16 if args.dtype == "f16" else torch.bfloat16
-    q, kc, vc, bt, ctx, slots, k_new, v_new = device_inputs(w, torch, dev, dt)
-    # like the reference's filler, the workload generator knows the lengths on the host
-    chunk = (choose_split(w.context_lens, w.num_kv_heads, w.num_heads) if args.chunk is None
-             else args.chunk)
-    split_name = {0: "balanced", -1: "whole sequence per workgroup"}.get(chunk,
-                                                                        f"fixed chunk {chunk}")
-    kernel_name = {0: "paged_decode_balanced_kernel", -1: "paged_decode_whole_kernel"}.get(
-        chunk, "paged_decode_splitk_kernel")
-    ws = DecodeWorkspace.for_shape(w.batch, w.num_heads, w.head_dim, w.max_blocks, w.block_size,
-                                   w.num_kv_heads, dev, chunk)
-    out = torch.empty_like(q)
-    kflat = kc.view(-1, w.num_kv_heads, w.head_dim)
-    vflat = vc.view(-1, w.num_kv_heads, w.head_dim)
-
-    variant = _lib.NVJ_PHASE_VALU_PRODUCTS if args.products == "valu" else 0
-
-    def decode(phases=3):
-        paged_attention(q, kc, vc, bt, ctx, w.scale, w.block_size, chunk=chunk, out=out,
-                        workspace=ws, phases=phases | variant)
-
-    def store():
-        store_kv_to_cache(k_new, v_new, kflat, vflat, slots)
+        lens = [int(x) for x in args.prefill_lens.split(",")]
+        print(json.dumps(prefill_record(lens, int(args.prefill_prefix), args.steps, args.warmup,
+                                        torch)), flush=True)
+        return 0
 
     if args.copy_calibration:
         src = torch.empty(1 << 30, dtype=torch.uint8, device=dev).fill_(1)
@@ -330,27 +444,27 @@ def main():
         torch.cuda.synchronize()
         del src, dst
 
-    store()
-    for _ in range(args.warmup):
-        decode()
-    ms_call, ms_wall = timed(decode, args.steps, torch)
-    ms_splitk, _ = timed(lambda: decode(_lib.NVJ_PHASE_SPLITK), args.steps, torch)
-    ms_combine, _ = timed(lambda: decode(_lib.NVJ_PHASE_COMBINE), args.steps, torch)
-    ms_store, _ = timed(store, args.steps, torch)
-    ms_graph = timed_in_graph(decode, torch)
-
-    byts = algorithmic_bytes(w.context_lens, w.batch, w.num_heads, w.num_kv_heads, w.head_dim,
-                             w.max_blocks)
-    gbps = byts / (ms_call * 1e-3) / 1e9
-    gbps_kernel = byts / (ms_splitk * 1e-3) / 1e9
+    chunk = args.chunk
+    m = decode_record(args.workload, chunk, args.dtype, args.products, args.steps, args.warmup,
+                      torch, dev, in_graph=True, keep_inputs=True)
+    w = m["workload"]
+    split_name = {0: "balanced", -1: "whole sequence per workgroup"}.get(chunk,
+                                                                        f"fixed chunk {chunk}")
+    kernel_name = {0: "paged_decode_balanced_kernel", -1: "paged_decode_whole_kernel"}.get(
+        chunk, "paged_decode_splitk_kernel")
+    byts = m["bytes"]
+    gbps = byts / (m["ms_call"] * 1e-3) / 1e9
+    gbps_kernel = byts / (m["ms_kernel"] * 1e-3) / 1e9
+    traffic, traffic_source = PROFILED_TRAFFIC.get((w.name, chunk, args.dtype, args.products),
+                                                   (None, None))
     rec = {
         "metric": "paged decode attn HBM GB/s (us/call alongside), Qwen3-8B shape B=64 ctx4k"
                   if w.name == "C2" else f"paged decode attn HBM GB/s, workload {w.name}",
         "value": round(gbps, 1), "unit": "GB/s", "n_gpus": 1, "steps": args.steps,
-        "warmup": args.warmup, "ms_per_step": round(ms_wall, 5), "higher_is_better": True,
+        "warmup": args.warmup, "ms_per_step": round(m["ms_wall"], 5), "higher_is_better": True,
         "scaling": "weak", "vs_baseline": None, "dtype": args.dtype, "data": "synthetic",
-        "us_per_call": round(ms_call * 1e3, 2),
-        "us_per_call_in_graph": round(ms_graph * 1e3, 2),
+        "us_per_call": round(m["ms_call"] * 1e3, 2),
+        "us_per_call_in_graph": round(m["ms_graph"] * 1e3, 2),
         "pct_of_hbm_peak": round(100.0 * gbps / HBM_PEAK_GBPS, 2),
         "config": {"workload": f"{w.name}: B={w.batch} Hq={w.num_heads} Hkv={w.num_kv_heads} "
                                f"D={w.head_dim} page={w.block_size} "
@@ -358,21 +472,27 @@ def main():
                                f"pool={w.num_blocks} pages",
                    "split": split_name, "products": args.products,
                    "algorithmic_bytes_per_call": byts,
-                   "step": "one launch" if chunk == -1 else "split-K launch + combine launch"},
+                   "step": "split-K launch + combine launch" if chunk > 0 else "one launch"},
         "roofline": {"bound": "hbm", "achieved": round(gbps_kernel, 1), "peak": HBM_PEAK_GBPS,
                      "unit": "GB/s", "frac": round(gbps_kernel / HBM_PEAK_GBPS, 4),
-                     "traffic": (MEASURED_TRAFFIC_BYTES.get((w.name, chunk))
-                                 if args.products == "mfma" else None),
+                     # not measured by this run: the counter figure of an earlier
+                     # profile of this configuration, with the file it is in
+                     "traffic": traffic, "traffic_source": traffic_source,
                      "kernel": kernel_name,
-                     "kernel_us": round(ms_splitk * 1e3, 2)},
-        # back-to-back launches of these two short kernels are paced by the host
-        # (one Python -> ctypes call each), not by the kernels themselves
-        "host_paced_launch_us": {"paged_decode_combine_kernel":
-                                 None if chunk == -1 else round(ms_combine * 1e3, 2),
-                                 "store_kvcache_kernel": round(ms_store * 1e3, 2)},
+                     "kernel_us": round(m["ms_kernel"] * 1e3, 2)},
+        # eager launches of this short kernel are paced by the host binding (one
+        # Python -> ctypes call each); inside a graph only the kernel remains
+        "store_kvcache_us": {"host_paced": round(m["ms_store"] * 1e3, 2),
+                             "in_graph": round(m["ms_store_graph"] * 1e3, 2)},
     }
+    q, kc, vc = m.pop("inputs")
     if not args.no_cpu_baseline:
         rec["cpu_baseline"] = cpu_baseline(w, q, kc, vc, args.cpu_budget, args.dtype)
+    # (freed blocks stay with torch's allocator on purpose: memory handed back to
+    # the driver and mapped again has measured 3-6 % slower for these kernels)
+    del q, kc, vc, m
+    if not args.no_others:
+        rec["others"] = others_block(args, torch, dev)
     print(json.dumps(rec), flush=True)
     return 0
 

@@ -55,8 +55,16 @@ What pins each function (see tests/test_oracle_pinning.py):
                                   expression is PARITY UNPINNED (at most one bf16
                                   ulp per rounding point).
 * ``paged_attention_fallback_ref``
-                                - same checks; the bf16 rounding of the
-                                  probabilities inside ``jax.nn.dot_product_attention``
+                                - the checks of the decode restatements above
+                                  (float64 brute force, torch SDPA with
+                                  ``enable_gqa``, ctx 0 / 1, equal keys, group
+                                  mapping, page permutation, padding and garbage,
+                                  one position more, out-of-range metadata), and a
+                                  float64 computation that rounds the
+                                  probabilities to bf16 at the same place, to one
+                                  bf16 ulp, on lengths 1 to 5 and across a page
+                                  boundary.  The rounding of the probabilities
+                                  inside ``jax.nn.dot_product_attention``
                                   (third-party jax, not under the reference
                                   tree, ``requirements.txt`` pins ``jax>=0.4.20``)
                                   is restated from its published XLA
@@ -279,7 +287,9 @@ def paged_decode_attention_per_seq_ref(q, k_cache, v_cache, block_tables,
     to_f32, to_bits = _codec(dtype)
     out = np.zeros((B, Hq, D), dtype=np.float32)
     for b in range(B):
-        n = int(ctx[b])
+        # the reference masks over the MB * bs gathered positions (:216-217): a
+        # length beyond them means all of them, a negative one none
+        n = min(int(ctx[b]), bt.shape[1] * block_size)
         if n <= 0:
             continue
         nblk = -(-n // block_size)

@@ -133,6 +133,67 @@ def test_reference_smoke_shape_b64():
     assert_close_bf16(got, want, what="reference smoke shape")
 
 
+def _fallback_case(name):
+    from nanovllm_jax_amd.workloads import draw_bf16_bits, make_workload
+    if name == "C1":
+        w = make_workload("C1")
+        rng = np.random.Generator(np.random.PCG64(w.seed + 200))
+        shape = (w.num_blocks, w.block_size, w.num_kv_heads, w.head_dim)
+        return (draw_bf16_bits(rng, (w.batch, w.num_heads, w.head_dim)),
+                draw_bf16_bits(rng, shape), draw_bf16_bits(rng, shape), w.block_tables,
+                w.context_lens, w.scale, w.block_size)
+    if name == "parity_d64":      # layers/pallas_attention.py:622-647
+        B, Hq, Hkv, D, bs, NB = 4, 8, 2, 64, 256, 32
+        bt = np.arange(16, dtype=np.int32).reshape(4, 4)
+        ctx = np.array([200, 512, 300, 100], np.int32)
+    else:                         # test_mosaic_kernels.py:30-54
+        B, Hq, Hkv, D, bs, NB = 64, 32, 8, 128, 256, 128
+        bt = (np.arange(B * 8, dtype=np.int32).reshape(B, 8) % NB).astype(np.int32)
+        ctx = np.minimum(200 + 50 * np.arange(B), 2048).astype(np.int32)
+    rng = np.random.Generator(np.random.PCG64(4200 + B))
+    return (draw_bf16_bits(rng, (B, Hq, D)), draw_bf16_bits(rng, (NB, bs, Hkv, D)),
+            draw_bf16_bits(rng, (NB, bs, Hkv, D)), bt, ctx, float(1.0 / np.sqrt(D)), bs)
+
+
+@pytest.mark.parametrize("chunk", [0, 256, -1])
+@pytest.mark.parametrize("name", ["C1", "parity_d64", "smoke_b64"])
+def test_against_the_fallback_oracle(name, chunk):
+    """The reference's second dispatch target - gather + dot_product_attention
+    (layers/attention.py:399-434), the one a jaxlib without Pallas takes - restated by
+    paged_attention_fallback_ref: bf16 operands, fp32 softmax, probabilities rounded to
+    bf16 before P.V.  Config C1, the shape of the reference's own parity check and the
+    shape of its decode smoke test, in every split mode."""
+    print(f"case fallback oracle {name} chunk={chunk}", flush=True)
+    from oracle.paged_attention_oracle import paged_attention_fallback_ref
+    q, kc, vc, bt, ctx, scale, bs = _fallback_case(name)
+    got = run_hip(q, kc, vc, bt, ctx, scale, bs, chunk)
+    want = paged_attention_fallback_ref(q, kc, vc, bt, ctx, scale, bs)
+    assert_close_bf16(got, want, what=f"fallback oracle {name} chunk={chunk}")
+
+
+@pytest.mark.parametrize("chunk", [0, 64, -1])
+def test_out_of_range_metadata_is_clamped_like_the_reference(chunk):
+    """A length beyond the table's reach means every described position, a negative one
+    gives zeros, live table entries below 0 or beyond the pool are clipped into it
+    (pallas_attention.py:185, :216-217): never a read outside the cache."""
+    print(f"case out-of-range metadata chunk={chunk}", flush=True)
+    from oracle.paged_attention_oracle import paged_decode_attention_vectorized_ref
+    B, Hq, Hkv, D, bs, NB = 6, 16, 8, 128, 64, 40
+    q, kc, vc, bt, ctx = make_problem(72, B, Hq, Hkv, D, bs, NB, [256, 256, 70, 200, 256, 100])
+    ctx = ctx.copy(); bt = bt.copy()
+    ctx[0] = 100000
+    ctx[1] = -3
+    bt[2, 0] = -1
+    bt[3, 1] = NB + 5
+    bt[4, 3] = 2 ** 30
+    bt[5, 1] = -(2 ** 31)
+    scale = float(1.0 / np.sqrt(D))
+    got = run_hip(q, kc, vc, bt, ctx, scale, bs, chunk)
+    want = paged_decode_attention_vectorized_ref(q, kc, vc, bt, ctx, scale, bs)
+    assert_close_bf16(got, want, what=f"out-of-range metadata chunk={chunk}")
+    assert not got[1].any()
+
+
 @pytest.mark.parametrize("B,seed", [(70, 1), (300, 2), (517, 3)])
 def test_balanced_split_many_ragged_sequences(B, seed):
     """The balanced split (chunk=0) derives its cut from context_lens on the

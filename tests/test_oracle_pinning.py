@@ -18,7 +18,10 @@ IMPLS = {
     "vectorized": lambda *a: bf16_bits_to_f32(paged_decode_attention_vectorized_ref(*a)),
     "per_seq": lambda *a: paged_decode_attention_per_seq_ref(*a, return_f32=True),
     "c": lambda *a: c_oracle.paged_decode(*a, return_f32=True),
+    "fallback": lambda *a: bf16_bits_to_f32(paged_attention_fallback_ref(*a)),
 }
+# these two return values rounded to bf16 (the fallback also rounds its probabilities)
+ROUNDED = ("vectorized", "fallback")
 
 
 # ---------------------------------------------------------------- bf16 rounding
@@ -111,7 +114,7 @@ def test_attention_against_fp64_brute_force(impl, Hq, Hkv):
     scale = 0.37
     want = textbook_attention_f64(q, kc, vc, bt, ctx, scale, bs)
     got = IMPLS[impl](q, kc, vc, bt, ctx, scale, bs)
-    tol = 1e-2 if impl == "vectorized" else 2e-5      # vectorized returns bf16-rounded values
+    tol = 1e-2 if impl in ROUNDED else 2e-5
     np.testing.assert_allclose(got, want, atol=tol, rtol=tol)
 
 
@@ -131,7 +134,7 @@ def test_attention_against_torch_sdpa_gqa(impl):
         o = torch.nn.functional.scaled_dot_product_attention(
             qq[None, :, None, :], k.permute(1, 0, 2)[None], v.permute(1, 0, 2)[None],
             scale=float(scale), enable_gqa=True)[0, :, 0, :].numpy()
-        tol = 1e-2 if impl == "vectorized" else 2e-5
+        tol = 1e-2 if impl in ROUNDED else 2e-5
         np.testing.assert_allclose(got[b], o, atol=tol, rtol=tol)
 
 
@@ -149,7 +152,7 @@ def test_attention_closed_forms(impl):
     v0 = bf16_bits_to_f32(vc[bt[1, 0], 0])                            # ctx = 1 -> V row
     np.testing.assert_allclose(got[1], np.repeat(v0, G, axis=0), rtol=1e-6, atol=0)
     v = bf16_bits_to_f32(vc[bt[2, :nblk]].reshape(-1, Hkv, D)[: ctx[2]]).astype(np.float64)
-    tol = 1e-2 if impl == "vectorized" else 1e-5
+    tol = 1e-2 if impl in ROUNDED else 1e-5
     np.testing.assert_allclose(got[2], np.repeat(v.mean(axis=0), G, axis=0), atol=tol, rtol=tol)
     # identical queries inside a group -> identical outputs
     q2 = q.copy(); q2[3, 1] = q2[3, 0]
@@ -184,6 +187,78 @@ def test_attention_layout_invariances(impl):
     # one position more really changes the answer (mask is not off by one)
     ctx4 = ctx.copy(); ctx4[0] += 1
     assert not np.allclose(IMPLS[impl](q, kc, vc, bt, ctx4, scale, bs)[0], base[0])
+
+
+def _f64_attention_with_rounded_probabilities(q, kc, vc, bt, ctx, scale, bs):
+    """float64 softmax, probabilities rounded to bf16, float64 P.V: what the fallback
+    computes, with every step but the one rounding exact."""
+    B, Hq, D = q.shape
+    Hkv = kc.shape[2]
+    G = Hq // Hkv
+    out = np.zeros((B, Hq, D))
+    for b in range(B):
+        n = int(ctx[b])
+        if n == 0:
+            continue
+        nblk = -(-n // bs)
+        k = bf16_bits_to_f32(kc[bt[b, :nblk]].reshape(-1, Hkv, D)[:n]).astype(np.float64)
+        v = bf16_bits_to_f32(vc[bt[b, :nblk]].reshape(-1, Hkv, D)[:n]).astype(np.float64)
+        for h in range(Hq):
+            s = k[:, h // G] @ bf16_bits_to_f32(q[b, h]).astype(np.float64) * scale
+            p = np.exp(s - s.max())
+            p /= p.sum()
+            p = bf16_bits_to_f32(f32_to_bf16_bits(p.astype(np.float32))).astype(np.float64)
+            out[b, h] = p @ v[:, h // G]
+    return out
+
+
+@pytest.mark.parametrize("Hq,Hkv", [(4, 4), (8, 2), (8, 1)])
+def test_fallback_against_float64_with_the_same_rounding_step(Hq, Hkv):
+    """Tighter than the 1e-2 bar: with the probabilities rounded to bf16 in an otherwise
+    exact float64 computation, the fallback restatement must agree to one bf16 ulp of the
+    result (its own final rounding) plus fp32 round-off.  Lengths 1 to 5 and a page
+    boundary: a mask off by one moves such a short row by far more."""
+    B, D, bs, NB = 8, 16, 8, 20
+    ctx = [1, 2, 3, 4, 5, 8, 9, 30]
+    q, kc, vc, bt, ctx = make_problem(61 + Hq, B, Hq, Hkv, D, bs, NB, ctx)
+    scale = 0.41
+    want = _f64_attention_with_rounded_probabilities(q, kc, vc, bt, ctx, scale, bs)
+    got = bf16_bits_to_f32(paged_attention_fallback_ref(q, kc, vc, bt, ctx, scale, bs))
+    # a probability that lands on the other side of a bf16 tie in fp32 moves the result by
+    # at most 2^-9 of that probability's share: allow 2^-7 relative, 2^-9 absolute
+    np.testing.assert_allclose(got, want, rtol=2.0 ** -7, atol=2.0 ** -9)
+    # and without the rounding step the agreement is visibly worse at these sizes
+    exact = textbook_attention_f64(q, kc, vc, bt, ctx, scale, bs)
+    assert np.abs(got - exact).max() > np.abs(got - want).max()
+
+
+def _bad_metadata_problem():
+    """Lengths beyond what the table describes and below zero, live table entries of -1
+    and beyond the pool: the literal restatement defines the result (clip of the table,
+    pallas_attention.py:185; mask over the MB * bs gathered positions, :216-217)."""
+    B, Hq, Hkv, D, bs, NB = 5, 8, 2, 16, 8, 16
+    q, kc, vc, bt, ctx = make_problem(71, B, Hq, Hkv, D, bs, NB, [24, 24, 9, 17, 24])
+    ctx = ctx.copy(); bt = bt.copy()
+    ctx[0] = 1000          # > MB * bs = 24: every gathered position is live
+    ctx[1] = -5            # nothing is live: zeros
+    bt[2, 0] = -1          # clipped to page 0
+    bt[3, 1] = NB + 7      # clipped to page NB - 1
+    bt[4, 2] = 2 ** 30
+    return q, kc, vc, bt, ctx, 0.3, bs
+
+
+@pytest.mark.parametrize("impl", ["per_seq", "c", "fallback"])
+def test_out_of_range_metadata_follows_the_literal_restatement(impl):
+    q, kc, vc, bt, ctx, scale, bs = _bad_metadata_problem()
+    want = bf16_bits_to_f32(paged_decode_attention_vectorized_ref(q, kc, vc, bt, ctx, scale, bs))
+    got = IMPLS[impl](q, kc, vc, bt, ctx, scale, bs)
+    np.testing.assert_allclose(got, want, atol=1e-2, rtol=1e-2)
+    assert not got[1].any()
+    # and the literal restatement itself against float64 on the clipped, clamped problem
+    NB = kc.shape[0]
+    exact = textbook_attention_f64(q, kc, vc, np.clip(bt, 0, NB - 1),
+                                   np.clip(ctx, 0, bt.shape[1] * bs), scale, bs)
+    np.testing.assert_allclose(want, exact, atol=1e-2, rtol=1e-2)
 
 
 def test_restatements_agree_with_each_other_at_c1():
