@@ -4,11 +4,17 @@
  *
  * Every entry point takes plain device pointers, sizes and a HIP stream
  * (passed as void* so the header needs no HIP include), only ENQUEUES work on
- * that stream, never synchronises, never allocates, keeps no global mutable
- * state and is re-entrant.  Return value: 0 on success, a negative NVJ_ERR_*
- * code otherwise (never throws, never exits).  Citations name the reference
- * interface each entry point stands in for (paths relative to the reference
- * checkout).
+ * that stream, never synchronises, never allocates and is re-entrant: the
+ * library keeps no state between calls other than two per-device look-ups it
+ * makes once (the number of compute units, the address of the array behind
+ * nvj_paged_decode_static_launch) and that array itself.  Return value: 0 on
+ * success, a negative NVJ_ERR_* code otherwise (never throws, never exits); the
+ * code reflects this call only (a launch reports its own status and does not
+ * read or clear the calling thread's HIP last-error slot).  Data pointers
+ * (q, out, caches, K/V rows, workspace, activations) must be 16-byte aligned,
+ * int32 metadata 4-byte aligned: NVJ_ERR_ALIGNMENT otherwise, from every entry
+ * point.  Citations name the reference interface each entry point stands in
+ * for (paths relative to the reference checkout).
  */
 #ifndef NVJ_PAGED_ATTN_H_
 #define NVJ_PAGED_ATTN_H_
@@ -31,7 +37,7 @@ extern "C" {
 #define NVJ_ERR_BAD_SHAPE     -2   /* negative size, Hq % Hkv != 0, ...             */
 #define NVJ_ERR_UNSUPPORTED   -3   /* head_dim / group size / block size not built  */
 #define NVJ_ERR_WORKSPACE     -4   /* workspace missing or too small                */
-#define NVJ_ERR_LAUNCH        -5   /* hipGetLastError() != hipSuccess after launch  */
+#define NVJ_ERR_LAUNCH        -5   /* the kernel launch itself reported an error     */
 #define NVJ_ERR_BAD_DTYPE     -6   /* unknown element type code                     */
 #define NVJ_ERR_SCRATCH_LIMIT -7   /* nvj_paged_decode_static_launch: the problem needs
                                       more than NVJ_STATIC_SCRATCH_BYTES of scratch  */

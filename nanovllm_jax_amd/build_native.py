@@ -81,7 +81,13 @@ def build_xla_ffi(verbose: bool = True) -> str | None:
            "-L", NATIVE_DIR, "-lnvj_paged_attn", "-Wl,-rpath,$ORIGIN", "-o", out]
     if verbose:
         print("[build]", " ".join(cmd), flush=True)
-    subprocess.run(cmd, check=True)
+    # this source has never met a compiler where it was written: a failure here
+    # must not take the rest of the build (and every test behind it) down
+    proc = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    if proc.returncode != 0:
+        print(f"[build] XLA FFI handlers did NOT compile (exit {proc.returncode}); the C-ABI "
+              f"library is unaffected:\n{proc.stdout}", flush=True)
+        return None
     return out
 
 

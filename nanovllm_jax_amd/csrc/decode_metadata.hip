@@ -14,6 +14,7 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include "launch.h"
 #include "nvj_paged_attn.h"
 
 namespace {
@@ -67,13 +68,13 @@ extern "C" int nvj_advance_decode_launch(void* stream, const void* next_tokens,
   if (max_blocks > 0 && !block_tables) return NVJ_ERR_NULL_POINTER;
   hipStream_t s = static_cast<hipStream_t>(stream);
   const dim3 grid((unsigned)((batch + 255) / 256)), block(256);
-  if (token_bytes == 8)
-    advance_decode_kernel<int64_t><<<grid, block, 0, s>>>(
-        static_cast<const int64_t*>(next_tokens), input_ids, positions, context_lens, slot_mapping,
-        block_tables, batch, max_blocks, block_size);
-  else
-    advance_decode_kernel<int32_t><<<grid, block, 0, s>>>(
-        static_cast<const int32_t*>(next_tokens), input_ids, positions, context_lens, slot_mapping,
-        block_tables, batch, max_blocks, block_size);
-  return hipGetLastError() == hipSuccess ? NVJ_OK : NVJ_ERR_LAUNCH;
+  const hipError_t rc =
+      token_bytes == 8
+          ? nvj::launch(advance_decode_kernel<int64_t>, grid, block, s,
+                        static_cast<const int64_t*>(next_tokens), input_ids, positions,
+                        context_lens, slot_mapping, block_tables, batch, max_blocks, block_size)
+          : nvj::launch(advance_decode_kernel<int32_t>, grid, block, s,
+                        static_cast<const int32_t*>(next_tokens), input_ids, positions,
+                        context_lens, slot_mapping, block_tables, batch, max_blocks, block_size);
+  return rc == hipSuccess ? NVJ_OK : NVJ_ERR_LAUNCH;
 }

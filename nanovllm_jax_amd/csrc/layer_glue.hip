@@ -20,6 +20,7 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include "launch.h"
 #include "nvj_paged_attn.h"
 
 namespace {
@@ -153,18 +154,15 @@ __global__ __launch_bounds__(256) void silu_and_mul_kernel(const uint4* __restri
 }
 
 template <int PIECES>
-void launch_add_rms_norm(hipStream_t stream, const uint4* x, const uint4* residual,
+hipError_t launch_add_rms_norm(hipStream_t stream, const uint4* x, const uint4* residual,
                          const float* weight, float eps, uint4* y, uint4* residual_out,
                          int num_tokens, int row_pieces) {
   const dim3 grid((unsigned)((num_tokens + 3) / 4)), block(256);
   if (residual != nullptr)
-    add_rms_norm_kernel<PIECES, true><<<grid, block, 0, stream>>>(x, residual, weight, eps, y,
-                                                                  residual_out, num_tokens,
-                                                                  row_pieces);
-  else
-    add_rms_norm_kernel<PIECES, false><<<grid, block, 0, stream>>>(x, nullptr, weight, eps, y,
-                                                                   nullptr, num_tokens,
-                                                                   row_pieces);
+    return nvj::launch(add_rms_norm_kernel<PIECES, true>, grid, block, stream, x, residual, weight,
+                       eps, y, residual_out, num_tokens, row_pieces);
+  return nvj::launch(add_rms_norm_kernel<PIECES, false>, grid, block, stream, x, nullptr, weight,
+                     eps, y, nullptr, num_tokens, row_pieces);
 }
 
 }  // namespace
@@ -188,12 +186,13 @@ extern "C" int nvj_add_rms_norm_launch(void* stream, const void* x, const void* 
   const auto rp = static_cast<const uint4*>(residual);
   const auto yp = static_cast<uint4*>(y);
   const auto op = static_cast<uint4*>(residual_out);
-  if (per_lane <= 1) launch_add_rms_norm<1>(s, xp, rp, weight, eps, yp, op, num_tokens, row_pieces);
-  else if (per_lane <= 2) launch_add_rms_norm<2>(s, xp, rp, weight, eps, yp, op, num_tokens, row_pieces);
-  else if (per_lane <= 4) launch_add_rms_norm<4>(s, xp, rp, weight, eps, yp, op, num_tokens, row_pieces);
-  else if (per_lane <= 8) launch_add_rms_norm<8>(s, xp, rp, weight, eps, yp, op, num_tokens, row_pieces);
-  else launch_add_rms_norm<16>(s, xp, rp, weight, eps, yp, op, num_tokens, row_pieces);
-  return hipGetLastError() == hipSuccess ? NVJ_OK : NVJ_ERR_LAUNCH;
+  hipError_t rc;
+  if (per_lane <= 1) rc = launch_add_rms_norm<1>(s, xp, rp, weight, eps, yp, op, num_tokens, row_pieces);
+  else if (per_lane <= 2) rc = launch_add_rms_norm<2>(s, xp, rp, weight, eps, yp, op, num_tokens, row_pieces);
+  else if (per_lane <= 4) rc = launch_add_rms_norm<4>(s, xp, rp, weight, eps, yp, op, num_tokens, row_pieces);
+  else if (per_lane <= 8) rc = launch_add_rms_norm<8>(s, xp, rp, weight, eps, yp, op, num_tokens, row_pieces);
+  else rc = launch_add_rms_norm<16>(s, xp, rp, weight, eps, yp, op, num_tokens, row_pieces);
+  return rc == hipSuccess ? NVJ_OK : NVJ_ERR_LAUNCH;
 }
 
 extern "C" int nvj_silu_and_mul_launch(void* stream, const void* x, int64_t x_row_stride, void* y,
@@ -208,8 +207,9 @@ extern "C" int nvj_silu_and_mul_launch(void* stream, const void* x, int64_t x_ro
   const int out_pieces = intermediate / 8;
   const int64_t blocks = ((int64_t)num_tokens * out_pieces + 255) / 256;
   if (blocks > INT32_MAX) return NVJ_ERR_BAD_SHAPE;
-  silu_and_mul_kernel<<<dim3((unsigned)blocks), dim3(256), 0, static_cast<hipStream_t>(stream)>>>(
+  const hipError_t rc = nvj::launch(
+      silu_and_mul_kernel, dim3((unsigned)blocks), dim3(256), static_cast<hipStream_t>(stream),
       static_cast<const uint4*>(x), x_row_stride / 8, static_cast<uint4*>(y), num_tokens,
       out_pieces);
-  return hipGetLastError() == hipSuccess ? NVJ_OK : NVJ_ERR_LAUNCH;
+  return rc == hipSuccess ? NVJ_OK : NVJ_ERR_LAUNCH;
 }

@@ -37,6 +37,7 @@
 
 #include <atomic>
 
+#include "launch.h"
 #include "nvj_paged_attn.h"
 
 namespace {
@@ -1570,14 +1571,15 @@ int launch_decode(void* stream, const void* q, const void* k_cache, const void* 
     if ((int64_t)batch * num_kv_heads > INT32_MAX) return NVJ_ERR_BAD_SHAPE;
     if (!(phases & NVJ_PHASE_SPLITK)) return NVJ_OK;   // there is no second pass
     const int hpw = heads_per_workgroup(batch, num_kv_heads);
-    const dim3 grid((unsigned)(batch * (num_kv_heads / hpw)));
-    if (valu && group == 4) paged_decode_whole_kernel<8, 128, false, 4><<<grid, dim3(512), 0, s>>>(a, hpw);
-    else if (valu) paged_decode_whole_kernel<8, 128, false, 8><<<grid, dim3(512), 0, s>>>(a, hpw);
-    else if (head_dim == 128 && !f16) paged_decode_whole_kernel<8, 128, false><<<grid, dim3(512), 0, s>>>(a, hpw);
-    else if (head_dim == 128) paged_decode_whole_kernel<8, 128, true><<<grid, dim3(512), 0, s>>>(a, hpw);
-    else if (!f16) paged_decode_whole_kernel<8, 64, false><<<grid, dim3(512), 0, s>>>(a, hpw);
-    else paged_decode_whole_kernel<8, 64, true><<<grid, dim3(512), 0, s>>>(a, hpw);
-    return hipGetLastError() == hipSuccess ? NVJ_OK : NVJ_ERR_LAUNCH;
+    const dim3 grid((unsigned)(batch * (num_kv_heads / hpw))), block(512);
+    hipError_t rc;
+    if (valu && group == 4) rc = nvj::launch(paged_decode_whole_kernel<8, 128, false, 4>, grid, block, s, a, hpw);
+    else if (valu) rc = nvj::launch(paged_decode_whole_kernel<8, 128, false, 8>, grid, block, s, a, hpw);
+    else if (head_dim == 128 && !f16) rc = nvj::launch(paged_decode_whole_kernel<8, 128, false>, grid, block, s, a, hpw);
+    else if (head_dim == 128) rc = nvj::launch(paged_decode_whole_kernel<8, 128, true>, grid, block, s, a, hpw);
+    else if (!f16) rc = nvj::launch(paged_decode_whole_kernel<8, 64, false>, grid, block, s, a, hpw);
+    else rc = nvj::launch(paged_decode_whole_kernel<8, 64, true>, grid, block, s, a, hpw);
+    return rc == hipSuccess ? NVJ_OK : NVJ_ERR_LAUNCH;
   }
 
   WorkspacePlan plan = {0, 1, 0, 0, 0, 0};
@@ -1596,14 +1598,16 @@ int launch_decode(void* stream, const void* q, const void* k_cache, const void* 
       // one launch: the workgroup that completes a sequence merges it
       if (phases & NVJ_PHASE_CLEAR_COUNTERS) {
         const int n = batch * num_kv_heads;
-        zero_int32_kernel<<<dim3((unsigned)((n + 255) / 256)), dim3(256), 0, s>>>(counters, n);
-        if (hipGetLastError() != hipSuccess) return NVJ_ERR_LAUNCH;
+        if (nvj::launch(zero_int32_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), s,
+                        counters, n) != hipSuccess)
+          return NVJ_ERR_LAUNCH;
       }
       if (!(phases & NVJ_PHASE_SPLITK)) return NVJ_OK;
       const dim3 grid((unsigned)plan.num_wgs);
-#define NVJ_LAUNCH_BALANCED(DV, F16V, VGV)                                      \
-  paged_decode_balanced_kernel<DV, F16V, VGV><<<grid, dim3(512), 0, s>>>(      \
-      a, batch, plan.num_wgs, kMinBalancedSteps, plan.hpw, counters)
+      hipError_t rc;
+#define NVJ_LAUNCH_BALANCED(DV, F16V, VGV)                                                     \
+  rc = nvj::launch(paged_decode_balanced_kernel<DV, F16V, VGV>, grid, dim3(512), s, a, batch, \
+                   plan.num_wgs, kMinBalancedSteps, plan.hpw, counters)
       if (valu && group == 4) NVJ_LAUNCH_BALANCED(128, false, 4);
       else if (valu) NVJ_LAUNCH_BALANCED(128, false, 8);
       else if (head_dim == 128 && !f16) NVJ_LAUNCH_BALANCED(128, false, 0);
@@ -1611,22 +1615,19 @@ int launch_decode(void* stream, const void* q, const void* k_cache, const void* 
       else if (!f16) NVJ_LAUNCH_BALANCED(64, false, 0);
       else NVJ_LAUNCH_BALANCED(64, true, 0);
 #undef NVJ_LAUNCH_BALANCED
-      return hipGetLastError() == hipSuccess ? NVJ_OK : NVJ_ERR_LAUNCH;
+      return rc == hipSuccess ? NVJ_OK : NVJ_ERR_LAUNCH;
     }
 
     if (phases & NVJ_PHASE_SPLITK) {
       const int nw = waves_per_workgroup(num_kv_heads);
       const dim3 grid((unsigned)(batch * plan.max_chunks), (unsigned)(num_kv_heads / nw));
       // one instantiation per (waves per workgroup, head_dim, element type)
-#define NVJ_LAUNCH_FIXED(NWV, DV)                                                             \
-  do {                                                                                        \
-    if (f16)                                                                                  \
-      paged_decode_splitk_kernel<NWV, DV, true><<<grid, dim3(NWV * 64), 0, s>>>(a, chunk,     \
-                                                                                plan.max_chunks); \
-    else                                                                                      \
-      paged_decode_splitk_kernel<NWV, DV, false><<<grid, dim3(NWV * 64), 0, s>>>(a, chunk,    \
-                                                                                 plan.max_chunks); \
-  } while (0)
+      hipError_t rc;
+#define NVJ_LAUNCH_FIXED(NWV, DV)                                                              \
+  rc = f16 ? nvj::launch(paged_decode_splitk_kernel<NWV, DV, true>, grid, dim3(NWV * 64), s, a, \
+                         chunk, plan.max_chunks)                                               \
+           : nvj::launch(paged_decode_splitk_kernel<NWV, DV, false>, grid, dim3(NWV * 64), s, a, \
+                         chunk, plan.max_chunks)
       switch (nw * 1000 + head_dim) {
         case 8128: NVJ_LAUNCH_FIXED(8, 128); break;
         case 4128: NVJ_LAUNCH_FIXED(4, 128); break;
@@ -1638,16 +1639,17 @@ int launch_decode(void* stream, const void* q, const void* k_cache, const void* 
         default: NVJ_LAUNCH_FIXED(1, 64); break;
       }
 #undef NVJ_LAUNCH_FIXED
-      if (hipGetLastError() != hipSuccess) return NVJ_ERR_LAUNCH;
+      if (rc != hipSuccess) return NVJ_ERR_LAUNCH;
     }
   } else {
     chunk = kStep;  // no pages at all: every sequence is empty, the second pass writes zeros
   }
   if (!(phases & NVJ_PHASE_COMBINE)) return NVJ_OK;
-  paged_decode_combine_kernel<<<dim3((unsigned)batch, (unsigned)num_heads), dim3(head_dim), 0, s>>>(
+  const hipError_t rc = nvj::launch(
+      paged_decode_combine_kernel, dim3((unsigned)batch, (unsigned)num_heads), dim3(head_dim), s,
       a.part_o, a.part_ml, context_lens, static_cast<uint16_t*>(out), num_heads, chunk,
       plan.max_chunks, max_blocks * block_size, a.scale_log2e, f16);
-  return hipGetLastError() == hipSuccess ? NVJ_OK : NVJ_ERR_LAUNCH;
+  return rc == hipSuccess ? NVJ_OK : NVJ_ERR_LAUNCH;
 }
 
 }  // namespace

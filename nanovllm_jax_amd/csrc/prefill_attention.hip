@@ -31,6 +31,7 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include "launch.h"
 #include "nvj_paged_attn.h"
 
 namespace {
@@ -545,11 +546,12 @@ int launch_prefill(hipStream_t stream, PrefillArgs a, bool paged, int32_t total_
   const dim3 grid((unsigned)((items + 7) / 8 * 8)), block(kWaves * 64);
   const int nt = (int)tiles;
   const bool f16 = dtype == NVJ_DTYPE_F16;
-  if (paged && f16) prefill_attention_kernel<true, true><<<grid, block, 0, stream>>>(a, nt);
-  else if (paged) prefill_attention_kernel<false, true><<<grid, block, 0, stream>>>(a, nt);
-  else if (f16) prefill_attention_kernel<true, false><<<grid, block, 0, stream>>>(a, nt);
-  else prefill_attention_kernel<false, false><<<grid, block, 0, stream>>>(a, nt);
-  return hipGetLastError() == hipSuccess ? NVJ_OK : NVJ_ERR_LAUNCH;
+  hipError_t rc;
+  if (paged && f16) rc = nvj::launch(prefill_attention_kernel<true, true>, grid, block, stream, a, nt);
+  else if (paged) rc = nvj::launch(prefill_attention_kernel<false, true>, grid, block, stream, a, nt);
+  else if (f16) rc = nvj::launch(prefill_attention_kernel<true, false>, grid, block, stream, a, nt);
+  else rc = nvj::launch(prefill_attention_kernel<false, false>, grid, block, stream, a, nt);
+  return rc == hipSuccess ? NVJ_OK : NVJ_ERR_LAUNCH;
 }
 
 }  // namespace

@@ -23,6 +23,7 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include "launch.h"
 #include "nvj_paged_attn.h"
 
 namespace {
@@ -124,10 +125,11 @@ extern "C" int nvj_qk_norm_rope_store_launch(void* stream, const void* qkv, int6
   const int64_t units = (int64_t)num_tokens * heads_total;
   const int64_t blocks = (units + 3) / 4;
   if (blocks > INT32_MAX) return NVJ_ERR_BAD_SHAPE;
-  qk_norm_rope_store_kernel<<<dim3((unsigned)blocks), dim3(256), 0, static_cast<hipStream_t>(stream)>>>(
-      static_cast<const uint16_t*>(qkv), qkv_row_stride, positions, cos_sin_cache, max_position,
+  const hipError_t rc = nvj::launch(
+      qk_norm_rope_store_kernel, dim3((unsigned)blocks), dim3(256),
+      static_cast<hipStream_t>(stream), static_cast<const uint16_t*>(qkv), qkv_row_stride, positions, cos_sin_cache, max_position,
       q_norm_weight, k_norm_weight, eps, slot_mapping, static_cast<uint16_t*>(k_cache),
       static_cast<uint16_t*>(v_cache), static_cast<uint16_t*>(q_out), num_tokens, num_heads,
       num_kv_heads, num_slots);
-  return hipGetLastError() == hipSuccess ? NVJ_OK : NVJ_ERR_LAUNCH;
+  return rc == hipSuccess ? NVJ_OK : NVJ_ERR_LAUNCH;
 }

@@ -11,6 +11,7 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include "launch.h"
 #include "nvj_paged_attn.h"
 
 namespace {
@@ -103,9 +104,10 @@ extern "C" int nvj_store_kvcache_launch(void* stream, const void* key, const voi
   uint4* vc = static_cast<uint4*>(v_cache);
   const bool kf = k_dtype == NVJ_DTYPE_F32, vf = v_dtype == NVJ_DTYPE_F32;
   const bool cf16 = cache_dtype == NVJ_DTYPE_F16;
-#define NVJ_LAUNCH_STORE(KF, VF, CF)                                                          \
-  store_kvcache_kernel<KF, VF, CF><<<grid, block, 0, s>>>(key, value, kc, vc, slot_mapping,   \
-                                                          num_tokens, pieces, num_slots)
+  hipError_t rc;
+#define NVJ_LAUNCH_STORE(KF, VF, CF)                                                      \
+  rc = nvj::launch(store_kvcache_kernel<KF, VF, CF>, grid, block, s, key, value, kc, vc, \
+                   slot_mapping, num_tokens, pieces, num_slots)
   switch ((kf ? 4 : 0) | (vf ? 2 : 0) | (cf16 ? 1 : 0)) {
     case 0: NVJ_LAUNCH_STORE(false, false, false); break;   // copies: the type does not matter
     case 1: NVJ_LAUNCH_STORE(false, false, false); break;
@@ -117,5 +119,5 @@ extern "C" int nvj_store_kvcache_launch(void* stream, const void* key, const voi
     default: NVJ_LAUNCH_STORE(true, true, true); break;
   }
 #undef NVJ_LAUNCH_STORE
-  return hipGetLastError() == hipSuccess ? NVJ_OK : NVJ_ERR_LAUNCH;
+  return rc == hipSuccess ? NVJ_OK : NVJ_ERR_LAUNCH;
 }

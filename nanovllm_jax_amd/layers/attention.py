@@ -33,27 +33,26 @@ def _require(cond: bool, msg: str) -> None:
         raise ValueError(msg)
 
 
-def store_kv_to_cache(key, value, k_cache, v_cache, slot_mapping):
-    """Scatter new K/V rows into the paged cache through ``slot_mapping``.
+def _raw_stream(device_index: int) -> int:
+    """The current HIP stream of a device as an integer handle."""
+    try:
+        return torch._C._cuda_getCurrentRawStream(device_index)
+    except AttributeError:      # a torch without the raw accessor
+        return torch.cuda.current_stream(device_index).cuda_stream
 
-    key, value   [num_tokens, num_kv_heads, head_dim], the cache dtype or float32
-                 (float32 rows are rounded to nearest even, as ``astype`` does)
-    k_cache, v_cache
-                 [num_slots, num_kv_heads, head_dim] bf16 or float16, or the 4-D
-                 [num_blocks, block_size, num_kv_heads, head_dim] view of the
-                 same memory
-    slot_mapping [num_tokens] int32; ``slot < 0`` skips the token, ``slot >=
-                 num_slots`` drops it
 
-    Returns ``(k_cache, v_cache)``: the tensors passed in, updated in place.
-    """
-    lib = _lib.load()
+# What a call signature (shapes, dtypes, devices of the five tensors) was validated
+# to: the integer arguments of the launch.  Validation is by far the larger part of
+# an eager call of this 3-microsecond kernel, so it runs once per signature.
+_store_plans: dict = {}
+
+
+def _plan_store(key, value, k_cache, v_cache, slot_mapping):
     for name, t in (("key", key), ("value", value), ("k_cache", k_cache),
                     ("v_cache", v_cache), ("slot_mapping", slot_mapping)):
         _require(isinstance(t, torch.Tensor), f"{name} must be a torch.Tensor")
         _require(t.is_cuda, f"{name} must live on the GPU (got {t.device}); "
                             "the KV-cache store has no CPU implementation")
-        _require(t.is_contiguous(), f"{name} must be contiguous")
         _require(t.device == key.device, f"{name} is on {t.device}, key on {key.device}")
     _require(key.dim() == 3 and value.shape == key.shape,
              "key and value must both be [num_tokens, num_kv_heads, head_dim]")
@@ -72,13 +71,53 @@ def store_kv_to_cache(key, value, k_cache, v_cache, slot_mapping):
     _require(slot_mapping.dtype == torch.int32 and slot_mapping.shape == (num_tokens,),
              "slot_mapping must be int32 [num_tokens]")
     num_slots = k_cache.numel() // (num_kv_heads * head_dim)
-    with torch.cuda.device(key.device):
-        stream = torch.cuda.current_stream(key.device).cuda_stream
-        code = lib.nvj_store_kvcache_launch(
-            stream, key.data_ptr(), value.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(),
-            slot_mapping.data_ptr(), num_tokens, num_kv_heads, head_dim, num_slots,
+    return (key.device.index, num_tokens, num_kv_heads, head_dim, num_slots,
             _DTYPE_CODE[key.dtype], _DTYPE_CODE[value.dtype], _DTYPE_CODE[k_cache.dtype])
-    _lib.check(code, "nvj_store_kvcache_launch")
+
+
+def store_kv_to_cache(key, value, k_cache, v_cache, slot_mapping):
+    """Scatter new K/V rows into the paged cache through ``slot_mapping``.
+
+    key, value   [num_tokens, num_kv_heads, head_dim], the cache dtype or float32
+                 (float32 rows are rounded to nearest even, as ``astype`` does)
+    k_cache, v_cache
+                 [num_slots, num_kv_heads, head_dim] bf16 or float16, or the 4-D
+                 [num_blocks, block_size, num_kv_heads, head_dim] view of the
+                 same memory
+    slot_mapping [num_tokens] int32; ``slot < 0`` skips the token, ``slot >=
+                 num_slots`` drops it
+
+    Returns ``(k_cache, v_cache)``: the tensors passed in, updated in place.
+    """
+    try:
+        sig = (key.shape, key.dtype, key.device, value.shape, value.dtype, value.device,
+               k_cache.shape, k_cache.dtype, k_cache.device, v_cache.shape, v_cache.dtype,
+               v_cache.device, slot_mapping.shape, slot_mapping.dtype, slot_mapping.device)
+    except AttributeError as e:
+        raise ValueError("store_kv_to_cache takes torch tensors") from e
+    plan = _store_plans.get(sig)
+    if plan is None:
+        plan = _plan_store(key, value, k_cache, v_cache, slot_mapping)
+        if len(_store_plans) < 256:
+            _store_plans[sig] = plan
+    # layout is a property of the tensor, not of the signature
+    if not (key.is_contiguous() and value.is_contiguous() and k_cache.is_contiguous()
+            and v_cache.is_contiguous() and slot_mapping.is_contiguous()):
+        raise ValueError("key, value, k_cache, v_cache and slot_mapping must be contiguous")
+    dev, num_tokens, num_kv_heads, head_dim, num_slots, kd, vd, cd = plan
+    if torch.cuda.current_device() == dev:
+        code = _lib.load().nvj_store_kvcache_launch(
+            _raw_stream(dev), key.data_ptr(), value.data_ptr(), k_cache.data_ptr(),
+            v_cache.data_ptr(), slot_mapping.data_ptr(), num_tokens, num_kv_heads, head_dim,
+            num_slots, kd, vd, cd)
+    else:
+        with torch.cuda.device(dev):
+            code = _lib.load().nvj_store_kvcache_launch(
+                _raw_stream(dev), key.data_ptr(), value.data_ptr(), k_cache.data_ptr(),
+                v_cache.data_ptr(), slot_mapping.data_ptr(), num_tokens, num_kv_heads, head_dim,
+                num_slots, kd, vd, cd)
+    if code != 0:
+        _lib.check(code, "nvj_store_kvcache_launch")
     return k_cache, v_cache
 
 

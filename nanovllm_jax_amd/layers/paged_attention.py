@@ -82,22 +82,91 @@ class DecodeWorkspace:
         return cls(need, device)
 
 
-def choose_split(context_lens_host, num_kv_heads: int, num_heads: int | None = None) -> int:
+def _compute_units(device=None) -> int:
+    """Compute units of a GPU (256 on an MI355X), asked once per device; 256 where
+    no GPU is visible (planning on a host without one)."""
+    if not torch.cuda.is_available():
+        return 256
+    index = torch.cuda.current_device() if device is None else torch.device(device).index
+    if index is None:
+        index = torch.cuda.current_device()
+    n = _CU_COUNT.get(index)
+    if n is None:
+        n = _CU_COUNT[index] = int(torch.cuda.get_device_properties(index).multi_processor_count)
+    return n
+
+
+_CU_COUNT: dict = {}
+
+
+def choose_split(context_lens_host, num_kv_heads: int, num_heads: int | None = None,
+                 device=None) -> int:
     """``chunk`` for a batch whose lengths the host knows (the reference's filler
     builds ``context_lens`` from Python ints, ``engine/model_runner.py:334-376``):
     ``WHOLE_SEQUENCE`` when the longest sequence is within 10 % of the mean and
-    the workgroups of that mode fill whole rounds of the 256 CUs to at least
-    95 % (one 8-wave workgroup is resident per CU), else 0 (balanced split)."""
+    the workgroups of that mode fill whole rounds of the GPU's compute units to at
+    least 95 % (one 8-wave workgroup is resident per CU), else 0 (balanced split,
+    which is never more than a few percent behind and right for any batch)."""
     lens = [int(n) for n in context_lens_host]
     if not lens:
         return 0
     mean = sum(lens) / len(lens)
     if mean <= 0 or max(lens) > 1.1 * mean:
         return 0
-    wgs = int(_lib.load().nvj_paged_decode_whole_sequence_workgroups(
+    cus = _compute_units(device)
+    count = lambda: int(_lib.load().nvj_paged_decode_whole_sequence_workgroups(
         len(lens), num_kv_heads if num_heads is None else num_heads, num_kv_heads))
-    rounds = -(-wgs // 256)
-    return WHOLE_SEQUENCE if wgs > 0 and wgs >= 0.95 * rounds * 256 else 0
+    if device is None:
+        wgs = count()
+    else:
+        with torch.cuda.device(device):     # the count follows the device's compute units
+            wgs = count()
+    rounds = -(-wgs // cus)
+    return WHOLE_SEQUENCE if wgs > 0 and wgs >= 0.95 * rounds * cus else 0
+
+
+def _raw_stream(device_index: int) -> int:
+    """The current HIP stream of a device as an integer handle."""
+    try:
+        return torch._C._cuda_getCurrentRawStream(device_index)
+    except AttributeError:      # a torch without the raw accessor
+        return torch.cuda.current_stream(device_index).cuda_stream
+
+
+# What a call signature (shapes, dtypes, devices, page size, split) was validated to:
+# the integer arguments of the launch and the workspace it needs.  Validation costs
+# several times the launch itself, so it runs once per signature.
+_decode_plans: dict = {}
+
+
+def _plan_decode(lib, q, k_cache, v_cache, block_tables, context_lens, block_size, chunk):
+    _check_device_tensor(q, "q", None, 3)
+    _check_device_tensor(k_cache, "k_cache", q.dtype, 4)
+    _check_device_tensor(v_cache, "v_cache", q.dtype, 4)
+    _check_device_tensor(block_tables, "block_tables", torch.int32, 2)
+    _check_device_tensor(context_lens, "context_lens", torch.int32, 1)
+    batch, num_heads, head_dim = q.shape
+    num_blocks, bs, num_kv_heads, d2 = k_cache.shape
+    _require(v_cache.shape == k_cache.shape, "k_cache and v_cache shapes differ")
+    _require(d2 == head_dim, f"head_dim mismatch: q {head_dim}, cache {d2}")
+    _require(int(block_size) == bs, f"block_size {block_size} != k_cache.shape[1] {bs}")
+    _require(block_tables.shape[0] == batch, "block_tables batch mismatch")
+    _require(context_lens.shape[0] == batch, "context_lens batch mismatch")
+    _require(num_heads % num_kv_heads == 0, "num_heads must be a multiple of num_kv_heads")
+    max_blocks = block_tables.shape[1]
+    dev = q.device
+    for name, t in (("k_cache", k_cache), ("v_cache", v_cache),
+                    ("block_tables", block_tables), ("context_lens", context_lens)):
+        _require(t.device == dev, f"{name} is on {t.device}, q on {dev}")
+    need = counters = 0
+    if batch and max_blocks:
+        with torch.cuda.device(dev):      # the balanced sizes follow the device's CU count
+            need = int(lib.nvj_paged_decode_workspace_bytes(batch, num_heads, head_dim,
+                                                            max_blocks, bs, num_kv_heads, chunk))
+            if chunk == 0:
+                counters = int(lib.nvj_paged_decode_counter_bytes(batch, num_heads, num_kv_heads))
+    return (dev.index, batch, num_heads, num_kv_heads, head_dim, bs, max_blocks, num_blocks, need,
+            counters, _CACHE_DTYPE_CODE[q.dtype])
 
 
 def paged_attention(q, k_cache, v_cache, block_tables, context_lens, scale, block_size,
@@ -125,60 +194,64 @@ def paged_attention(q, k_cache, v_cache, block_tables, context_lens, scale, bloc
     have; ``phases`` selects the launches (timing aid).
     """
     lib = _lib.load()
-    _check_device_tensor(q, "q", None, 3)
-    _check_device_tensor(k_cache, "k_cache", q.dtype, 4)
-    _check_device_tensor(v_cache, "v_cache", q.dtype, 4)
-    _check_device_tensor(block_tables, "block_tables", torch.int32, 2)
-    _check_device_tensor(context_lens, "context_lens", torch.int32, 1)
-    batch, num_heads, head_dim = q.shape
-    num_blocks, bs, num_kv_heads, d2 = k_cache.shape
-    _require(v_cache.shape == k_cache.shape, "k_cache and v_cache shapes differ")
-    _require(d2 == head_dim, f"head_dim mismatch: q {head_dim}, cache {d2}")
-    _require(int(block_size) == bs, f"block_size {block_size} != k_cache.shape[1] {bs}")
-    _require(block_tables.shape[0] == batch, "block_tables batch mismatch")
-    _require(context_lens.shape[0] == batch, "context_lens batch mismatch")
-    _require(num_heads % num_kv_heads == 0, "num_heads must be a multiple of num_kv_heads")
-    max_blocks = block_tables.shape[1]
+    try:
+        sig = (q.shape, q.dtype, q.device, k_cache.shape, k_cache.dtype, k_cache.device,
+               v_cache.shape, v_cache.dtype, v_cache.device, block_tables.shape,
+               block_tables.dtype, block_tables.device, context_lens.shape, context_lens.dtype,
+               context_lens.device, int(block_size), int(chunk))
+    except AttributeError as e:
+        raise ValueError("paged_attention takes torch tensors") from e
+    plan = _decode_plans.get(sig)
+    if plan is None:
+        plan = _plan_decode(lib, q, k_cache, v_cache, block_tables, context_lens, block_size,
+                            chunk)
+        if len(_decode_plans) < 256:
+            _decode_plans[sig] = plan
+    # layout is a property of the tensor, not of the signature
+    _require(q.is_contiguous() and k_cache.is_contiguous() and v_cache.is_contiguous()
+             and block_tables.is_contiguous() and context_lens.is_contiguous(),
+             "q, k_cache, v_cache, block_tables and context_lens must be contiguous")
+    (dev_index, batch, num_heads, num_kv_heads, head_dim, bs, max_blocks, num_blocks, need,
+     counters, dtype_code) = plan
     dev = q.device
-    for name, t in (("k_cache", k_cache), ("v_cache", v_cache),
-                    ("block_tables", block_tables), ("context_lens", context_lens)):
-        _require(t.device == dev, f"{name} is on {t.device}, q on {dev}")
 
     if out is None:
         out = torch.empty_like(q)
     else:
-        _check_device_tensor(out, "out", q.dtype, 3)
-        _require(out.shape == q.shape and out.device == dev, "out must match q")
-    need = int(lib.nvj_paged_decode_workspace_bytes(batch, num_heads, head_dim, max_blocks,
-                                                    bs, num_kv_heads, chunk)) if batch and max_blocks else 0
+        _require(isinstance(out, torch.Tensor) and out.dtype == q.dtype and out.shape == q.shape
+                 and out.device == dev and out.is_contiguous(),
+                 "out must be a contiguous tensor matching q")
+    phases = int(phases)
     if isinstance(workspace, DecodeWorkspace):
         # its counters are zero between calls, unless a call of a smaller shape
         # has since written partials where this call's counters lie
-        counters = int(lib.nvj_paged_decode_counter_bytes(batch, num_heads, num_kv_heads)) \
-            if chunk == 0 and batch and max_blocks else 0
         if counters > workspace.zero_prefix:
-            phases = int(phases) | _lib.NVJ_PHASE_CLEAR_COUNTERS
-        if chunk >= 0 and batch and max_blocks:
+            phases |= _lib.NVJ_PHASE_CLEAR_COUNTERS
+        if chunk >= 0 and need:
             workspace.zero_prefix = counters
         workspace = workspace.buffer
     else:
-        phases = int(phases) | _lib.NVJ_PHASE_CLEAR_COUNTERS
+        phases |= _lib.NVJ_PHASE_CLEAR_COUNTERS
     if workspace is None:
         workspace = torch.empty(max(need, 16), dtype=torch.uint8, device=dev)
     else:
         _require(workspace.is_cuda and workspace.device == dev and workspace.is_contiguous(),
                  "workspace must be a contiguous tensor on q's device")
-        _require(workspace.numel() * workspace.element_size() >= need,
-                 f"workspace too small: need {need} bytes")
     ws_bytes = workspace.numel() * workspace.element_size()
+    _require(ws_bytes >= need, f"workspace too small: need {need} bytes")
 
-    with torch.cuda.device(dev):
-        stream = torch.cuda.current_stream(dev).cuda_stream
-        code = lib.nvj_paged_decode_launch_phases(
-            stream, q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(),
+    def launch():
+        return lib.nvj_paged_decode_launch_phases(
+            _raw_stream(dev_index), q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(),
             block_tables.data_ptr(), context_lens.data_ptr(), out.data_ptr(),
             workspace.data_ptr(), ws_bytes, batch, num_heads, num_kv_heads, head_dim, bs,
-            max_blocks, num_blocks, float(scale), int(chunk), _CACHE_DTYPE_CODE[q.dtype],
-            int(phases))
-    _lib.check(code, "nvj_paged_decode_launch_phases")
+            max_blocks, num_blocks, float(scale), int(chunk), dtype_code, phases)
+
+    if torch.cuda.current_device() == dev_index:
+        code = launch()
+    else:
+        with torch.cuda.device(dev_index):
+            code = launch()
+    if code != 0:
+        _lib.check(code, "nvj_paged_decode_launch_phases")
     return out

@@ -2,9 +2,8 @@
 
 Host-side mirror of ``utils/context.py`` of the reference (``AttentionContext``
 :35-81, ``create_decode_context`` :169-190): same field names and meaning, with
-device tensors in place of JAX arrays.  Only the decode fields are populated by
-this package; the prefill fields exist so that code written against the
-reference's dataclass keeps working.
+device tensors in place of JAX arrays, for the decode phase and (``create_prefill_context``)
+the prefill phase.
 """
 from __future__ import annotations
 
@@ -15,24 +14,19 @@ __all__ = ["AttentionContext", "create_decode_context", "create_prefill_context"
 
 
 def _bucket_to_power_of_2(value: int, min_bucket: int = 16, max_bucket: int = 8192) -> int:
-    """Next power of two in [min_bucket, max_bucket] (``utils/context.py:18-32``:
-    the reference buckets its static max lengths to limit recompilation; kept so
-    that contexts carry the same values)."""
-    if value <= min_bucket:
-        return min_bucket
-    if value >= max_bucket:
-        return max_bucket
-    power = 1
-    while power < value:
-        power *= 2
-    return min(power, max_bucket)
+    """``value`` rounded up to a power of two and clamped into [min_bucket,
+    max_bucket]: what the reference's helper of this name returns
+    (``utils/context.py:18-32``; it buckets the static max lengths to limit
+    recompilation).  The HIP kernels never read these fields; the contexts carry
+    them so that code written against the reference sees the same values."""
+    return max(min_bucket, min(max_bucket, 1 << max(int(value) - 1, 0).bit_length()))
 
 
 @dataclass
 class AttentionContext:
     """Metadata one attention call needs.
 
-    is_prefill          False for decode (the only phase this package runs).
+    is_prefill          False for decode, True for prefill.
     context_lens        [batch] int32, length of every sequence including the
                         position being decoded.
     slot_mapping        [num_tokens] int32, cache slot of every new K/V row;
