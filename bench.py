@@ -37,7 +37,7 @@ HBM_PEAK_GBPS = 8000.0
 # 1 GiB copy.  Not measured by the run that prints them: reported with the file
 # they come from, and only for the exact configuration that was profiled.
 PROFILED_TRAFFIC = {
-    ("C2", 0, "bf16", "mfma"): (None, "profiles/paged_decode_balanced_kernel_C2.md"),
+    ("C2", 0, "bf16", "mfma"): (1_075_020_000, "profiles/paged_decode_balanced_kernel_C2.md"),
     ("C2", -1, "bf16", "mfma"): (1_074_909_000, "profiles/paged_decode_whole_kernel_C2.md"),
 }
 
@@ -300,7 +300,8 @@ def decode_record(name, chunk, dtype, products, steps, warmup, torch, dev, in_gr
     out = torch.empty_like(q)
     kflat = kc.view(-1, w.num_kv_heads, w.head_dim)
     vflat = vc.view(-1, w.num_kv_heads, w.head_dim)
-    variant = _lib.NVJ_PHASE_VALU_PRODUCTS if products == "valu" else 0
+    variant = {"valu": _lib.NVJ_PHASE_VALU_PRODUCTS, "none": _lib.NVJ_PHASE_LOADS_ONLY}.get(
+        products, 0)
 
     def decode(phases=_lib.NVJ_PHASE_SPLITK | _lib.NVJ_PHASE_COMBINE):
         paged_attention(q, kc, vc, bt, ctx, w.scale, w.block_size, chunk=chunk, out=out,
@@ -391,10 +392,11 @@ def main():
     ap.add_argument("--dtype", default="bf16", choices=["bf16", "f16"],
                     help="cache / q / out dtype; f16 is what the reference's own timing "
                          "scripts use")
-    ap.add_argument("--products", default="mfma", choices=["mfma", "valu"],
+    ap.add_argument("--products", default="mfma", choices=["mfma", "valu", "none"],
                     help="valu: time the measurement variant of the kernel that does "
                          "Q.K and P.V with vector-ALU dot products (group 4 or 8, bf16, "
-                         "balanced or whole-sequence split)")
+                         "balanced or whole-sequence split); none: the variant that only "
+                         "streams K and V (no arithmetic: the memory stream by itself)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-others", action="store_true",
                     help="skip the `others` block (the other workloads, prefill, decode step)")

@@ -218,11 +218,18 @@ NVJ_API int nvj_paged_decode_launch(void* stream,
  * Exists for head_dim 128, bf16, exactly 4 or 8 query heads per KV head, a
  * multiple of 8 KV heads and chunk 0 or NVJ_CHUNK_WHOLE_SEQUENCE; anything else
  * returns NVJ_ERR_UNSUPPORTED.
+ *
+ * NVJ_PHASE_LOADS_ONLY, or-ed in, runs a second measurement variant: the same
+ * page walk and K/V loads with no arithmetic behind them, so that the time of
+ * the memory stream alone can be set against the real kernel's.  `out` receives
+ * meaningless finite values.  head_dim 128, bf16, chunk 0 or
+ * NVJ_CHUNK_WHOLE_SEQUENCE; anything else returns NVJ_ERR_UNSUPPORTED.
  */
 #define NVJ_PHASE_SPLITK  1u
 #define NVJ_PHASE_COMBINE 2u
 #define NVJ_PHASE_VALU_PRODUCTS 4u
 #define NVJ_PHASE_CLEAR_COUNTERS 8u
+#define NVJ_PHASE_LOADS_ONLY 16u
 NVJ_API int nvj_paged_decode_launch_phases(void* stream,
                             const void* q, const void* k_cache, const void* v_cache,
                             const int32_t* block_tables, const int32_t* context_lens,

@@ -71,6 +71,7 @@ NVJ_PHASE_SPLITK = 1
 NVJ_PHASE_COMBINE = 2
 NVJ_PHASE_VALU_PRODUCTS = 4
 NVJ_PHASE_CLEAR_COUNTERS = 8
+NVJ_PHASE_LOADS_ONLY = 16
 
 _lock = threading.Lock()
 _lib = None

@@ -263,6 +263,12 @@ __device__ __forceinline__ void compute_segment(const DecodeArgs& a, uint4* lds,
     for (int i = 0; i < H::kKLoads; ++i)
       lds[(H::kPosPerLoad * i + lane / H::kPieces) * H::kLdsRowPieces + lane % H::kPieces] =
           kreg[i];
+    // Other lanes read these rows below.  The wave's own LDS accesses complete
+    // in order; the fences keep the compiler from moving the reads ahead of the
+    // writes (and, at the end of the step, the next writes ahead of the reads).
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
     if (more) {
       if (next_last == kStep - 1)
         issue_k_loads<false, D>(kreg, k_cache + next_off, lane, next_last, row_bytes);
@@ -352,6 +358,8 @@ __device__ __forceinline__ void compute_segment(const DecodeArgs& a, uint4* lds,
       acc[jd] *= alpha;
       acc[jd] = Elem<F16>::mfma(vt[jd], pbits, acc[jd]);
     }
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
   }
 
   // total of the running sum over the 4 k-groups that share column r
@@ -668,6 +676,69 @@ __device__ __forceinline__ void compute_segment_valu(const DecodeArgs& a, uint4*
   __builtin_amdgcn_wave_barrier();
 }
 
+// ---------------------------------------------------------------------------
+// Measurement variant: the load stream of a segment and nothing else.  Same
+// page walk, same K and V loads (addresses, order, one step fetched ahead) as
+// compute_segment, but what arrives is only folded into one word per lane: no
+// LDS, no matrix or softmax work.  Timing it against the real kernel shows how
+// much of the kernel's time the arithmetic adds on top of the memory stream.
+// The "result" is meaningless (and finite).  head_dim 128 only.
+// ---------------------------------------------------------------------------
+__device__ __forceinline__ void compute_segment_loads_only(const DecodeArgs& a, int b, int kvh,
+                                                           int t0, int t1, int lane,
+                                                           f32x4 (&acc)[8], float& m_run,
+                                                           float& l_run) {
+  constexpr int D = 128;
+  using H = HeadDim<D>;
+  const int r = lane & 15, kg = lane >> 4;
+  const int block_size = a.block_size, num_blocks = a.num_blocks;
+  const int nsteps = (t1 - t0 + kStep - 1) / kStep;
+  const uint32_t row_bytes = (uint32_t)a.cache_kv_heads * (D * 2);
+  const int64_t head_bytes = (int64_t)(kvh / a.kv_rep) * (D * 2);
+  const const_i32_ptr table = as_constant(a.block_tables + (int64_t)b * a.max_blocks);
+  auto step_base = [&](int step) -> int64_t {
+    const int ts = t0 + step * kStep;
+    const int page = ts / block_size;
+    const int phys = min(max(table[page], 0), num_blocks - 1);
+    return ((int64_t)phys * block_size + (ts - page * block_size)) * row_bytes + head_bytes;
+  };
+  uint4 kreg[H::kKLoads], vreg[8];
+  {
+    const int64_t off = step_base(0);
+    const int last = min(kStep, t1 - t0) - 1;
+    issue_k_loads<true, D>(kreg, a.k_cache + off, lane, last, row_bytes);
+    issue_v_loads<true, D>(vreg, a.v_cache + off, kg, r, last, row_bytes);
+  }
+#pragma unroll
+  for (int jd = 0; jd < 8; ++jd) acc[jd] = f32x4{0.f, 0.f, 0.f, 0.f};
+  m_run = 0.f;
+  l_run = 0.f;
+  uint32_t folded = 0;
+  int64_t off_ahead = nsteps > 1 ? step_base(1) : 0;
+  for (int step = 0; step < nsteps; ++step) {
+    const bool more = step + 1 < nsteps;
+    const int64_t next_off = off_ahead;
+    int next_last = kStep - 1;
+    if (more) next_last = min(kStep, t1 - (t0 + (step + 1) * kStep)) - 1;
+    if (step + 2 < nsteps) off_ahead = step_base(step + 2);
+#pragma unroll
+    for (int i = 0; i < H::kKLoads; ++i) folded ^= kreg[i].x ^ kreg[i].y ^ kreg[i].z ^ kreg[i].w;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) folded ^= vreg[j].x ^ vreg[j].y ^ vreg[j].z ^ vreg[j].w;
+    if (more) {
+      if (next_last == kStep - 1) {
+        issue_k_loads<false, D>(kreg, a.k_cache + next_off, lane, next_last, row_bytes);
+        issue_v_loads<false, D>(vreg, a.v_cache + next_off, kg, r, next_last, row_bytes);
+      } else {
+        issue_k_loads<true, D>(kreg, a.k_cache + next_off, lane, next_last, row_bytes);
+        issue_v_loads<true, D>(vreg, a.v_cache + next_off, kg, r, next_last, row_bytes);
+      }
+    }
+    l_run += 1.0f;
+  }
+  acc[0][0] = (float)(folded & 0xFFu);
+}
+
 // Normalised bf16 result of a whole sequence straight to `out`.
 template <int D, bool F16>
 __device__ __forceinline__ void write_output(const DecodeArgs& a, int b, int kvh, int lane,
@@ -742,7 +813,8 @@ __global__ __launch_bounds__(NW * 64) void paged_decode_splitk_kernel(DecodeArgs
 // wave's K tile is free by then and exactly holds its 34 floats per lane) and
 // the wave of part 0 merges them and writes the output.  Meant for batches of
 // similar lengths: a workgroup's time follows its sequence's length.
-// VG > 0 selects the vector-ALU measurement variant for exactly VG query heads
+// VG < 0 selects the loads-only measurement variant; VG > 0 selects the
+// vector-ALU measurement variant for exactly VG query heads
 // per KV head (head_dim 128, bf16 only).
 template <int NW, int D, bool F16, int VG = 0>
 __global__ __launch_bounds__(NW * 64) void paged_decode_whole_kernel(DecodeArgs a, int hpw) {
@@ -772,6 +844,9 @@ __global__ __launch_bounds__(NW * 64) void paged_decode_whole_kernel(DecodeArgs 
     if constexpr (VG > 0)
       compute_segment_valu<VG>(a, k_tile[wave], b, kvh, s0 * kStep, min(ctx, s1 * kStep), lane,
                                acc, m_run, l_run);
+    else if constexpr (VG < 0)
+      compute_segment_loads_only(a, b, kvh, s0 * kStep, min(ctx, s1 * kStep), lane, acc, m_run,
+                                 l_run);
     else
       compute_segment<D, F16>(a, k_tile[wave], b, kvh, s0 * kStep, min(ctx, s1 * kStep), lane,
                               acc, m_run, l_run);
@@ -1237,6 +1312,8 @@ __global__ __launch_bounds__(512) void paged_decode_balanced_kernel(DecodeArgs a
       const int t1 = __builtin_amdgcn_readfirstlane(min(ctx, en * kStep));
       if constexpr (VG > 0)
         compute_segment_valu<VG>(a, k_tile[wave], sb, kvh, t0, t1, lane, acc, m_run, l_run);
+      else if constexpr (VG < 0)
+        compute_segment_loads_only(a, sb, kvh, t0, t1, lane, acc, m_run, l_run);
       else
         compute_segment<D, F16>(a, k_tile[wave], sb, kvh, t0, t1, lane, acc, m_run, l_run);
       x += en - st;
@@ -1546,6 +1623,9 @@ int launch_decode(void* stream, const void* q, const void* k_cache, const void* 
   if (valu && (head_dim != 128 || f16 || kv_rep != 1 || (group != 4 && group != 8) ||
                num_kv_heads % 8 != 0 || chunk > 0))
     return NVJ_ERR_UNSUPPORTED;
+  // the loads-only measurement variant: head_dim 128, bf16, not with a fixed chunk
+  const bool loads_only = (phases & NVJ_PHASE_LOADS_ONLY) != 0;
+  if (loads_only && (valu || head_dim != 128 || f16 || chunk > 0)) return NVJ_ERR_UNSUPPORTED;
   hipStream_t s = static_cast<hipStream_t>(stream);
 
   DecodeArgs a;
@@ -1573,7 +1653,8 @@ int launch_decode(void* stream, const void* q, const void* k_cache, const void* 
     const int hpw = heads_per_workgroup(batch, num_kv_heads);
     const dim3 grid((unsigned)(batch * (num_kv_heads / hpw))), block(512);
     hipError_t rc;
-    if (valu && group == 4) rc = nvj::launch(paged_decode_whole_kernel<8, 128, false, 4>, grid, block, s, a, hpw);
+    if (loads_only) rc = nvj::launch(paged_decode_whole_kernel<8, 128, false, -1>, grid, block, s, a, hpw);
+    else if (valu && group == 4) rc = nvj::launch(paged_decode_whole_kernel<8, 128, false, 4>, grid, block, s, a, hpw);
     else if (valu) rc = nvj::launch(paged_decode_whole_kernel<8, 128, false, 8>, grid, block, s, a, hpw);
     else if (head_dim == 128 && !f16) rc = nvj::launch(paged_decode_whole_kernel<8, 128, false>, grid, block, s, a, hpw);
     else if (head_dim == 128) rc = nvj::launch(paged_decode_whole_kernel<8, 128, true>, grid, block, s, a, hpw);
@@ -1608,7 +1689,8 @@ int launch_decode(void* stream, const void* q, const void* k_cache, const void* 
 #define NVJ_LAUNCH_BALANCED(DV, F16V, VGV)                                                     \
   rc = nvj::launch(paged_decode_balanced_kernel<DV, F16V, VGV>, grid, dim3(512), s, a, batch, \
                    plan.num_wgs, kMinBalancedSteps, plan.hpw, counters)
-      if (valu && group == 4) NVJ_LAUNCH_BALANCED(128, false, 4);
+      if (loads_only) NVJ_LAUNCH_BALANCED(128, false, -1);
+      else if (valu && group == 4) NVJ_LAUNCH_BALANCED(128, false, 4);
       else if (valu) NVJ_LAUNCH_BALANCED(128, false, 8);
       else if (head_dim == 128 && !f16) NVJ_LAUNCH_BALANCED(128, false, 0);
       else if (head_dim == 128) NVJ_LAUNCH_BALANCED(128, true, 0);
