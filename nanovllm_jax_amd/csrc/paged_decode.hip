@@ -908,8 +908,9 @@ __device__ __forceinline__ int wave_inclusive_scan(int x) {
 // The unit of work is a "row step": one 32-position step of one row, a row
 // being (sequence b, head group hg of hpw KV heads).  All row steps, ordered
 // by (b, hg, step), form one axis of length T = (num_kv_heads / hpw) * sum of
-// steps.  The axis is cut into sub-runs of `lp` row steps, lp the same for
-// all: sub-run j = [j*lp, (j+1)*lp) belongs to workgroup j / R, part j % R, and
+// steps.  The axis is cut into `nsub` sub-runs of equal length to within one
+// step (`Cut` below): nsub = workgroups x R when there is at least one step for
+// each, fewer otherwise.  Sub-run j belongs to workgroup j / R, part j % R, and
 // is walked by the hpw waves of that part, one KV head each.  Every wave
 // derives the cut from context_lens itself (a wave-wide prefix sum over the
 // batch), so the host never needs the lengths.
@@ -920,7 +921,8 @@ __device__ __forceinline__ int wave_inclusive_scan(int x) {
 // along the axis, and consecutive within a row).  When the whole run of a
 // workgroup lies inside one row, its parts are first merged through LDS (a
 // wave's K tile is free by then) and part 0 writes one partial for all of
-// them; the other parts mark their slots empty (sum 0).
+// them; the slots of the other parts stay unused, which the merging wave knows
+// from the cut.
 //
 // Merge without a second launch: `counters` holds one int32 per (sequence, KV
 // head), zero between launches.  A wave that has written partials for a row
@@ -929,6 +931,25 @@ __device__ __forceinline__ int wave_inclusive_scan(int x) {
 // from the cut) merges the row's partials in slot order, writes the output and
 // puts the counter back to zero.  Nothing ever waits for another workgroup.
 // ---------------------------------------------------------------------------
+
+// The cut of the axis: sub-run j covers the axis positions whose unit
+// (position >> shift) lies in [floor(j * units / nsub), floor((j+1) * units / nsub)).
+// shift is 0 unless the axis is so long that units * nsub would not fit 31 bits
+// (the host picks it from the largest axis the shapes allow).  Every sub-run
+// holds at least one position.
+struct Cut {
+  int axis;    // row steps in all
+  int units;   // ceil(axis >> shift)
+  int nsub;    // sub-runs in use, 1 <= nsub <= units
+  int shift;
+  __device__ __forceinline__ int start_of(int j) const {
+    const uint32_t u = (uint32_t)j * (uint32_t)units / (uint32_t)nsub;
+    return min(axis, (int)(u << shift));
+  }
+  __device__ __forceinline__ int subrun_of(int x) const {
+    return (int)((((uint32_t)(x >> shift) + 1u) * (uint32_t)nsub - 1u) / (uint32_t)units);
+  }
+};
 
 // Record (see write_partial) of query head 0 of KV head `h_in_row` of a slot.
 __device__ __forceinline__ int64_t balanced_record(const DecodeArgs& a, int64_t slot, int hpw,
@@ -1000,14 +1021,14 @@ __device__ __forceinline__ void wait_for_stores() {
 // them.  merge_row: all partials of the row are there; merge them in slot order
 // and write the output.  `lds` is the wave's own tile (free at that point).
 //
-// The merge keeps the chain of dependent memory round trips short: the (max,
-// sum) pairs of 16 slots are fetched by four loads issued together and spread
-// to the lanes through LDS; empty slots are then skipped, and the accumulators
-// of two real partials are in flight at once.
+// The merge keeps the chain of dependent memory round trips short: which slots
+// hold a partial is computed from the cut, not read; the (max, sum) pairs of up
+// to 64 slots are fetched by loads issued together and spread to the lanes
+// through LDS; the accumulators of four partials are in flight at once.
 // Returns true when this arrival completed the row: the caller then owes the
 // row its merge (merge_row), at a time of its choosing.
 __device__ __forceinline__ bool arrive(const DecodeArgs& a, int32_t* counters, int b, int kvh,
-                                       int r0, int r1, int lp, int n, int lane) {
+                                       int r0, int r1, const Cut& cut, int n, int lane) {
   // the partial stores of every lane have reached the device before the count does
   wait_for_stores();
   int32_t* counter = counters + (int64_t)b * a.num_kv_heads + kvh;
@@ -1015,7 +1036,7 @@ __device__ __forceinline__ bool arrive(const DecodeArgs& a, int32_t* counters, i
   if (lane == 0)
     old = __hip_atomic_fetch_add(counter, n, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   old = __builtin_amdgcn_readfirstlane(old);
-  const int expected = (r1 - 1) / lp - r0 / lp + 1;
+  const int expected = cut.subrun_of(r1 - 1) - cut.subrun_of(r0) + 1;
   if (old + n != expected) return false;
   // last to arrive: every other partial of the row was acknowledged before its
   // writer's count, which this wave has just seen
@@ -1026,110 +1047,118 @@ __device__ __forceinline__ bool arrive(const DecodeArgs& a, int32_t* counters, i
 
 template <int D, bool F16>
 __device__ __forceinline__ void merge_row(const DecodeArgs& a, uint4* lds, int b, int kvh,
-                                          int hpw, int r0, int r1, int lp, int lane) {
-  const int first = r0 / lp;
-  const int expected = (r1 - 1) / lp - first + 1;
+                                          int hpw, int r0, int r1, const Cut& cut, int lane) {
+  using H = HeadDim<D>;
+  // slots whose (max, sum) pairs fit the wave's tile at 16 heads x 8 bytes each
+  constexpr int kSlots = (kStep * H::kLdsRowPieces * 16) / 128 >= 64 ? 64 : 32;
+  constexpr int KG = D / 32;
+  const int parts = 8 / hpw;
+  const int first = cut.subrun_of(r0);
+  const int expected = cut.subrun_of(r1 - 1) - first + 1;
   const int hg = kvh / hpw;
   const int rows_per_seq = a.num_kv_heads / hpw;
   const int64_t slot0 = (int64_t)first + (int64_t)b * rows_per_seq + hg;
   // lanes of padding heads / padding dims read a real record and drop it later
   const int r = min(lane & 15, a.group - 1);
   const int kg = (32 * (lane >> 4) < D) ? (lane >> 4) : 0;
-  constexpr int KG = D / 32;
   const int64_t rec0 = balanced_record(a, slot0, hpw, kvh - hg * hpw);   // slot0, head 0
   const int64_t rec_stride = (int64_t)hpw * a.group;                     // per slot
   const __amdgpu_buffer_rsrc_t wm = device_window(
       a.part_ml + rec0 * 2, ((int64_t)(expected - 1) * rec_stride + a.group) * 2 * sizeof(float));
   const int lane_off = (kg * a.group + r) * 16, piece_stride = KG * a.group * 16;
-  vfloat2* lds_ml = reinterpret_cast<vfloat2*>(lds);   // [16 slots][16 heads]
+  vfloat2* lds_ml = reinterpret_cast<vfloat2*>(lds);   // [kSlots][16 heads]
   f32x4 acc[8];
 #pragma unroll
   for (int jd = 0; jd < 8; ++jd) acc[jd] = f32x4{0.f, 0.f, 0.f, 0.f};
   float m_run = kNegBig, l_run = 0.f;
-  for (int base = 0; base < expected; base += 16) {
-    // (max, sum) of slots base .. base + 15 for the 16 head columns: lane (r, kg)
-    // fetches slot base + 4 * i + kg for i = 0 .. 3; slots past the end repeat the last
-    vfloat2 got[4];
+  for (int base = 0; base < expected; base += kSlots) {
+    // Which of the slots base .. base + kSlots - 1 hold a partial follows from the
+    // cut: lane L answers for slot base + L.  A workgroup whose whole run lies
+    // inside this row merged its parts in LDS and wrote one partial, in the slot
+    // of its part 0; any other workgroup wrote one per sub-run.
+    const int count = min(kSlots, expected - base);
+    const int j = first + base + lane;
+    const int g = j / parts;
+    const bool inside = cut.start_of(g * parts) >= r0 &&
+                        cut.start_of(min(cut.nsub, g * parts + parts)) <= r1;
+    unsigned long long real = __ballot(lane < count && (!inside || j == g * parts));
+    // (max, sum) of all these slots for the 16 head columns, the loads in flight
+    // together: lane (r, kg) fetches slot base + 4 * i + kg (unused slots hold
+    // stale values that are never looked at; slots past the end repeat the last).
+    // (Fetching them together with the accumulators of the first partials, one
+    // round trip fewer on paper, measured 2 us slower at 8 short sequences.)
+    vfloat2 got[kSlots / 4];
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
+    for (int i = 0; i < kSlots / 4; ++i) {
       const int s = min(base + 4 * i + (lane >> 4), expected - 1);
       got[i] = __builtin_bit_cast(vfloat2, __builtin_amdgcn_raw_buffer_load_b64(
                                                wm, (int)((s * rec_stride + r) * 8), 0, kDeviceScope));
     }
 #pragma unroll
-    for (int i = 0; i < 4; ++i) lds_ml[(4 * i + (lane >> 4)) * 16 + (lane & 15)] = got[i];
+    for (int i = 0; i < kSlots / 4; ++i) lds_ml[(4 * i + (lane >> 4)) * 16 + (lane & 15)] = got[i];
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
     __builtin_amdgcn_wave_barrier();
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-    const int count = min(16, expected - base);
-    // which of the slots hold a partial (sum > 0): the same for every head
-    uint32_t real = 0;
-    float m_chunk = kNegBig;
-#pragma unroll
-    for (int i = 0; i < 16; ++i) {
-      const vfloat2 x = lds_ml[i * 16 + (lane & 15)];
-      if (i < count && x.y > 0.f) {
-        real |= 1u << i;
-        m_chunk = fmaxf(m_chunk, x.x);
-      }
-    }
-    real = __builtin_amdgcn_readfirstlane(real);
-    if (real != 0u) {
+    if (real != 0ull) {
+      float m_chunk = kNegBig;
+      for (unsigned long long todo = real; todo != 0ull; todo &= todo - 1ull)
+        m_chunk = fmaxf(m_chunk, lds_ml[__builtin_ctzll(todo) * 16 + (lane & 15)].x);
       const float m_new = fmaxf(m_run, m_chunk);
       const float keep = __builtin_amdgcn_exp2f((m_run - m_new) * a.scale_log2e);
       m_run = m_new;
       l_run *= keep;
 #pragma unroll
       for (int jd = 0; jd < 8; ++jd) acc[jd] *= keep;
-      while (real != 0u) {
-        // two real partials at a time; an absent second repeats the first with weight 0
-        const int i0 = __builtin_ctz(real);
-        real &= real - 1u;
-        const bool two = real != 0u;
-        const int i1 = two ? __builtin_ctz(real) : i0;
-        if (two) real &= real - 1u;
-        const __amdgpu_buffer_rsrc_t win0 = device_window(
-            a.part_o + (rec0 + (base + i0) * rec_stride) * D, (int64_t)a.group * D * sizeof(float));
-        const __amdgpu_buffer_rsrc_t win1 = device_window(
-            a.part_o + (rec0 + (base + i1) * rec_stride) * D, (int64_t)a.group * D * sizeof(float));
-        vfloat4 v0[8], v1[8];
+      while (real != 0ull) {
+        // up to four partials at a time; absent ones repeat the first with weight 0
+        int idx[4];
+        float w[4];
+        vfloat4 v[4][8];
 #pragma unroll
-        for (int i = 0; i < 8; ++i)
-          v0[i] = __builtin_bit_cast(vfloat4, __builtin_amdgcn_raw_buffer_load_b128(
-                                                  win0, lane_off + i * piece_stride, 0, kDeviceScope));
+        for (int k = 0; k < 4; ++k) {
+          const bool have = real != 0ull;
+          idx[k] = have ? __builtin_ctzll(real) : idx[0];
+          if (have) real &= real - 1ull;
+          const __amdgpu_buffer_rsrc_t win =
+              device_window(a.part_o + (rec0 + (base + idx[k]) * rec_stride) * D,
+                            (int64_t)a.group * D * sizeof(float));
 #pragma unroll
-        for (int i = 0; i < 8; ++i)
-          v1[i] = __builtin_bit_cast(vfloat4, __builtin_amdgcn_raw_buffer_load_b128(
-                                                  win1, lane_off + i * piece_stride, 0, kDeviceScope));
-        const vfloat2 ml0 = lds_ml[i0 * 16 + (lane & 15)];
-        const vfloat2 ml1 = lds_ml[i1 * 16 + (lane & 15)];
-        const float w0 = __builtin_amdgcn_exp2f((ml0.x - m_new) * a.scale_log2e);
-        const float w1 = two ? __builtin_amdgcn_exp2f((ml1.x - m_new) * a.scale_log2e) : 0.f;
-        l_run = fmaf(w0, ml0.y, fmaf(w1, ml1.y, l_run));
-#pragma unroll
-        for (int e = 0; e < 4; ++e) {
-          acc[0][e] = fmaf(w0, v0[2 * e].x, fmaf(w1, v1[2 * e].x, acc[0][e]));
-          acc[1][e] = fmaf(w0, v0[2 * e].y, fmaf(w1, v1[2 * e].y, acc[1][e]));
-          acc[2][e] = fmaf(w0, v0[2 * e].z, fmaf(w1, v1[2 * e].z, acc[2][e]));
-          acc[3][e] = fmaf(w0, v0[2 * e].w, fmaf(w1, v1[2 * e].w, acc[3][e]));
-          acc[4][e] = fmaf(w0, v0[2 * e + 1].x, fmaf(w1, v1[2 * e + 1].x, acc[4][e]));
-          acc[5][e] = fmaf(w0, v0[2 * e + 1].y, fmaf(w1, v1[2 * e + 1].y, acc[5][e]));
-          acc[6][e] = fmaf(w0, v0[2 * e + 1].z, fmaf(w1, v1[2 * e + 1].z, acc[6][e]));
-          acc[7][e] = fmaf(w0, v0[2 * e + 1].w, fmaf(w1, v1[2 * e + 1].w, acc[7][e]));
+          for (int i = 0; i < 8; ++i)
+            v[k][i] = __builtin_bit_cast(
+                vfloat4, __builtin_amdgcn_raw_buffer_load_b128(win, lane_off + i * piece_stride, 0,
+                                                               kDeviceScope));
+          const vfloat2 ml = lds_ml[idx[k] * 16 + (lane & 15)];
+          w[k] = have ? __builtin_amdgcn_exp2f((ml.x - m_new) * a.scale_log2e) : 0.f;
+          l_run = fmaf(w[k], ml.y, l_run);
         }
+#pragma unroll
+        for (int k = 0; k < 4; ++k)
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            acc[0][e] = fmaf(w[k], v[k][2 * e].x, acc[0][e]);
+            acc[1][e] = fmaf(w[k], v[k][2 * e].y, acc[1][e]);
+            acc[2][e] = fmaf(w[k], v[k][2 * e].z, acc[2][e]);
+            acc[3][e] = fmaf(w[k], v[k][2 * e].w, acc[3][e]);
+            acc[4][e] = fmaf(w[k], v[k][2 * e + 1].x, acc[4][e]);
+            acc[5][e] = fmaf(w[k], v[k][2 * e + 1].y, acc[5][e]);
+            acc[6][e] = fmaf(w[k], v[k][2 * e + 1].z, acc[6][e]);
+            acc[7][e] = fmaf(w[k], v[k][2 * e + 1].w, acc[7][e]);
+          }
       }
     }
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-    __builtin_amdgcn_wave_barrier();   // the next chunk overwrites lds_ml
+    __builtin_amdgcn_wave_barrier();   // the next pass overwrites lds_ml
   }
   write_output<D, F16>(a, b, kvh, lane, acc, l_run);
 }
 
-// grid.x = num_wgs, block = 512.  `min_steps`: lower bound of lp.
+// grid.x = num_wgs, block = 512.  `min_steps`: fewest steps a sub-run may have
+// (in units of 1 << shift steps); `shift`: see Cut.
 template <int D, bool F16, int VG = 0>
 __global__ __launch_bounds__(512) void paged_decode_balanced_kernel(DecodeArgs a, int batch,
                                                                     int num_wgs, int min_steps,
-                                                                    int hpw, int32_t* counters) {
+                                                                    int hpw, int shift,
+                                                                    int32_t* counters) {
   using H = HeadDim<D>;
   constexpr int NW = 8;
   __shared__ uint4 k_tile[NW][kStep * H::kLdsRowPieces];
@@ -1190,12 +1219,15 @@ __global__ __launch_bounds__(512) void paged_decode_balanced_kernel(DecodeArgs a
         orow[i] = make_uint4(0u, 0u, 0u, 0u);
     }
   }
-  const int axis = rows_per_seq * total;   // T
-  const int lp = max(((axis + num_wgs - 1) / num_wgs + parts - 1) / parts, min_steps);
-  const int run = lp * parts;
-  const int start = g * run;
-  if (start >= axis) return;
-  const int end = min(axis, start + run);
+  Cut cut;
+  cut.axis = rows_per_seq * total;
+  cut.shift = shift;
+  cut.units = (cut.axis + (1 << shift) - 1) >> shift;
+  cut.nsub = max(1, min(num_wgs * parts, cut.units / min_steps));
+  if (cut.axis == 0 || g * parts >= cut.nsub) return;
+  const int nparts = min(parts, cut.nsub - g * parts);   // parts of this workgroup that have work
+  const int start = cut.start_of(g * parts);
+  const int end = cut.start_of(g * parts + nparts);
 
   // the sequence whose rows hold axis position x: its index, the steps before
   // it and its length (all wave-uniform)
@@ -1245,14 +1277,13 @@ __global__ __launch_bounds__(512) void paged_decode_balanced_kernel(DecodeArgs a
   const int nb0 = (ctx0 + kStep - 1) / kStep;
   const int hg0 = (start - rows_per_seq * before0) / nb0;
   const int row0 = rows_per_seq * before0 + hg0 * nb0;   // axis position of the row's step 0
-  const int xs = start + part * lp;
-  const int xe = min(end, xs + lp);
+  const int xs = part < nparts ? cut.start_of(g * parts + part) : end;
+  const int xe = part < nparts ? cut.start_of(g * parts + part + 1) : end;
   const int64_t subrun = (int64_t)g * parts + part;
   // Does the whole run of the workgroup lie inside one row?  Then every wave has
   // at most one segment, and the parts of a head meet in LDS before anything is
   // written.  Otherwise every wave walks its own sub-run across the rows.
   const bool single = end <= row0 + nb0;
-  const int nparts = (end - start + lp - 1) / lp;   // parts of this workgroup that have work
   if (!single && xs >= xe) return;
 
   int b = b0, before = before0, ctx = ctx0;
@@ -1261,20 +1292,6 @@ __global__ __launch_bounds__(512) void paged_decode_balanced_kernel(DecodeArgs a
   // lengths, page lookups and address arithmetic stay on the scalar unit.  The
   // guards (b inside the batch, x not before the sequence) cannot fire when
   // the prefix sums are right; they keep every index in range regardless.
-  if (single && part > 0 && xs < xe && !(start == row0 && end == row0 + nb0)) {
-    // Part 0 will carry this part's share in its own partial: this part's slot
-    // is marked empty (sum 0).  Stored now, so that the acknowledgement it must
-    // wait for before the parts meet arrives while the wave works.
-    if (lane < a.group) {
-      const int64_t rec =
-          balanced_record(a, subrun + (int64_t)b0 * rows_per_seq + hg0, hpw, h_in_row);
-      const __amdgpu_buffer_rsrc_t wm =
-          device_window(a.part_ml + rec * 2, (int64_t)a.group * 2 * sizeof(float));
-      const vfloat2 empty = {kNegBig, 0.f};
-      __builtin_amdgcn_raw_buffer_store_b64(__builtin_bit_cast(vuint2, empty), wm, lane * 8, 0,
-                                            kDeviceScope);
-    }
-  }
   int x = xs;
   int owed = 0, owed_b[2] = {0, 0}, owed_kvh[2] = {0, 0}, owed_row[2] = {0, 0}, owed_nb[2] = {1, 1};
   for (;;) {
@@ -1338,9 +1355,6 @@ __global__ __launch_bounds__(512) void paged_decode_balanced_kernel(DecodeArgs a
             mine[32 * kLanesWithDims] = m_run;
             mine[33 * kLanesWithDims] = l_run;
           }
-          // the empty marker stored before the work began has been acknowledged
-          // by now; part 0 publishes the count after the barrier below
-          if (!direct) wait_for_stores();
         }
         __syncthreads();
         if (part > 0) return;
@@ -1370,7 +1384,7 @@ __global__ __launch_bounds__(512) void paged_decode_balanced_kernel(DecodeArgs a
       const int64_t slot = subrun + (int64_t)sb * rows_per_seq + hg;
       write_partial_coherent<D>(a, balanced_record(a, slot, hpw, h_in_row), lane, acc, m_run,
                                 l_run);
-      if (arrive(a, counters, sb, kvh, row, row + nb, lp, covers, lane)) {
+      if (arrive(a, counters, sb, kvh, row, row + nb, cut, covers, lane)) {
         // at most the first and the last segment of a sub-run are not whole rows
         if (owed == 0) { owed_b[0] = sb; owed_kvh[0] = kvh; owed_row[0] = row; owed_nb[0] = nb; }
         else { owed_b[1] = sb; owed_kvh[1] = kvh; owed_row[1] = row; owed_nb[1] = nb; }
@@ -1385,7 +1399,7 @@ __global__ __launch_bounds__(512) void paged_decode_balanced_kernel(DecodeArgs a
     const int okvh = __builtin_amdgcn_readfirstlane(i == 0 ? owed_kvh[0] : owed_kvh[1]);
     const int orow = __builtin_amdgcn_readfirstlane(i == 0 ? owed_row[0] : owed_row[1]);
     const int onb = __builtin_amdgcn_readfirstlane(i == 0 ? owed_nb[0] : owed_nb[1]);
-    merge_row<D, F16>(a, k_tile[wave], ob, okvh, hpw, orow, orow + onb, lp, lane);
+    merge_row<D, F16>(a, k_tile[wave], ob, okvh, hpw, orow, orow + onb, cut, lane);
   }
 }
 
@@ -1507,7 +1521,7 @@ int waves_per_workgroup(int num_kv_heads) {
 struct WorkspacePlan {
   int64_t records;  // partial records (one query head each)
   int max_chunks;   // fixed-chunk mode only
-  int num_wgs, hpw; // balanced mode only
+  int num_wgs, hpw, shift; // balanced mode only
   size_t counter_bytes;
   size_t bytes;
 };
@@ -1525,6 +1539,9 @@ bool plan_workspace(int64_t batch, int64_t num_heads, int64_t head_dim, int64_t 
     wgs = wgs < 1 ? 1 : wgs > cus ? cus : wgs;
     plan->num_wgs = (int)wgs;
     plan->hpw = hpw;
+    // (units + 1) * sub-runs must fit 31 bits (Cut): coarser units for a very long axis
+    plan->shift = 0;
+    while ((((axis >> plan->shift) + 2) * wgs * parts) >> 31) ++plan->shift;
     plan->max_chunks = 0;
     const int64_t slots = wgs * parts + batch * rows_per_seq;
     plan->records = slots * hpw * (num_heads / num_kv_heads);
@@ -1534,7 +1551,7 @@ bool plan_workspace(int64_t batch, int64_t num_heads, int64_t head_dim, int64_t 
   }
   const int64_t mc = (max_blocks * block_size + chunk - 1) / chunk;
   if (batch * mc > INT32_MAX) return false;
-  plan->num_wgs = plan->hpw = 0;
+  plan->num_wgs = plan->hpw = plan->shift = 0;
   plan->max_chunks = (int)mc;
   plan->records = batch * mc * num_heads;
   plan->counter_bytes = 0;
@@ -1663,7 +1680,7 @@ int launch_decode(void* stream, const void* q, const void* k_cache, const void* 
     return rc == hipSuccess ? NVJ_OK : NVJ_ERR_LAUNCH;
   }
 
-  WorkspacePlan plan = {0, 1, 0, 0, 0, 0};
+  WorkspacePlan plan = {0, 1, 0, 0, 0, 0, 0};
   if (max_blocks > 0) {
     if (!plan_workspace(batch, num_heads, head_dim, max_blocks, block_size, num_kv_heads, chunk,
                         &plan))
@@ -1688,7 +1705,7 @@ int launch_decode(void* stream, const void* q, const void* k_cache, const void* 
       hipError_t rc;
 #define NVJ_LAUNCH_BALANCED(DV, F16V, VGV)                                                     \
   rc = nvj::launch(paged_decode_balanced_kernel<DV, F16V, VGV>, grid, dim3(512), s, a, batch, \
-                   plan.num_wgs, kMinBalancedSteps, plan.hpw, counters)
+                   plan.num_wgs, kMinBalancedSteps, plan.hpw, plan.shift, counters)
       if (loads_only) NVJ_LAUNCH_BALANCED(128, false, -1);
       else if (valu && group == 4) NVJ_LAUNCH_BALANCED(128, false, 4);
       else if (valu) NVJ_LAUNCH_BALANCED(128, false, 8);
