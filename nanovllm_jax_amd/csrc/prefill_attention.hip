@@ -14,8 +14,8 @@
 // 32 at a time.  The K rows and the V rows of a tile go from global memory
 // straight into LDS (global_load_lds_dwordx4: no staging registers, no LDS
 // write instructions), row-major with the 16-byte pieces of a row permuted so
-// that the reads below are free of bank conflicts, in rings of 3 (K) and 4 (V)
-// tiles fetched two tiles ahead; one barrier per tile:
+// that the reads below are free of bank conflicts, in rings of 4 tiles each,
+// fetched two tiles ahead; one barrier per tile:
 //   * K is read back with ds_read_b128 as the A operand of
 //     S^T[key, q] = K . Q^T  (v_mfma_f32_16x16x32_bf16, Q^T of both groups in
 //     registers for the whole tile);
@@ -50,8 +50,14 @@ constexpr int kRowsPerWave = 16 * kGroups;
 constexpr int kBM = kRowsPerWave * kWaves;   // query rows per workgroup
 constexpr int kKeys = 32;            // keys per step
 constexpr int kTileBytes = kKeys * kD * 2;   // one K or V tile in LDS: 32 rows of 256 bytes
-constexpr int kKStages = 3;          // K tiles i .. i+2 are live in iteration i
-constexpr int kVStages = 4;          // V tiles i-1 .. i+2
+// Both rings hold 4 tiles, tile t in slot t % 4: iteration i reads K of tile i and
+// V of tile i-1 while tiles i+1 (landing) and i+2 (just issued) are on their way.
+// A ring of 3 would do for K; 4 makes the slot of every tile of an iteration a
+// function of i % 4, so that a loop unrolled 4 times has every LDS offset as an
+// instruction immediate.
+constexpr int kKStages = 4;
+constexpr int kVStages = 4;
+constexpr int kStages = 4;
 constexpr float kNegBig = -1.0e30f;
 constexpr float kLazyLog2 = 8.0f;    // running max moves only for gains above 2^8
 constexpr float kLog2e = 1.4426950408889634f;
@@ -168,6 +174,38 @@ struct TileCopier {
                     v_lds + (uint32_t)v_stage * kTileBytes + dst);
     }
   }
+
+  // The same for a tile all of whose 32 keys exist (tile < last_tile): the
+  // lanes' offsets do not depend on the tile and are computed once (lane_offsets).
+  __device__ __forceinline__ void lane_offsets(uint32_t (&koff)[kCopyRowsPerWave / 4],
+                                               uint32_t (&voff)[kCopyRowsPerWave / 4]) const {
+#pragma unroll
+    for (int j = 0; j < kCopyRowsPerWave / 4; ++j) {
+      const int row = kCopyRowsPerWave * wave + 4 * j + (lane >> 4);
+      const uint32_t row_off = __umul24(row, row_bytes);
+      koff[j] = row_off + 16u * k_position(row, lane & 15);
+      voff[j] = row_off + 16u * v_position(row, lane & 15);
+    }
+  }
+  template <int STAGE>
+  __device__ __forceinline__ void issue_full(int tile, const uint32_t (&koff)[kCopyRowsPerWave / 4],
+                                             const uint32_t (&voff)[kCopyRowsPerWave / 4]) const {
+    const int ks = tile * kKeys;
+    size_t first_row = (size_t)ks;
+    if (PAGED) {
+      const int page = ks / block_size;
+      const int phys = min(max(table[page], 0), num_blocks - 1);
+      first_row = (size_t)phys * block_size + (ks - page * block_size);
+    }
+    const char* kb = k_head + first_row * row_bytes;
+    const char* vb = v_head + first_row * row_bytes;
+#pragma unroll
+    for (int j = 0; j < kCopyRowsPerWave / 4; ++j) {
+      const uint32_t dst = (uint32_t)(kCopyRowsPerWave / 4 * wave + j) * 1024u;
+      copy16_to_lds(kb, koff[j], k_lds + (uint32_t)STAGE * kTileBytes + dst);
+      copy16_to_lds(vb, voff[j], v_lds + (uint32_t)STAGE * kTileBytes + dst);
+    }
+  }
 };
 constexpr int kCopiesPerTile = 2 * (kCopyRowsPerWave / 4);   // copy16_to_lds calls of one lane per tile
 
@@ -195,16 +233,20 @@ __device__ __forceinline__ float max_of8(const f32x4& a, const f32x4& b) {
 
 // S^T of one 32-key tile against both column groups (16 query rows each):
 // sc[g][h] holds keys 16*h + 4*kg + e of the tile for query row r of group g.
+// kaddr[s] is the lane's LDS address of its piece 4*s + kg of row r of ring slot
+// 0 (k_read_addresses); `slot_bytes` selects the ring slot.
 template <bool F16>
-__device__ __forceinline__ void scores_of_tile(lds_ptr kt, const bf16x8 (&qreg)[kGroups][4],
-                                               f32x4 (&sc)[kGroups][2], int r, int kg) {
+__device__ __forceinline__ void scores_of_tile(const lds_ptr (&kaddr)[4], int slot_bytes,
+                                               const bf16x8 (&qreg)[kGroups][4],
+                                               f32x4 (&sc)[kGroups][2]) {
   bf16x8 ka[2][4];
 #pragma unroll
   for (int s = 0; s < 4; ++s) {
     // rows r and 16 + r share a position: (16 + r) & 15 == r
-    const int at = 256 * r + 16 * k_position(r, 4 * s + kg);
-    ka[0][s] = *reinterpret_cast<const __attribute__((address_space(3))) bf16x8*>(kt + at);
-    ka[1][s] = *reinterpret_cast<const __attribute__((address_space(3))) bf16x8*>(kt + at + 16 * 256);
+    ka[0][s] = *reinterpret_cast<const __attribute__((address_space(3))) bf16x8*>(
+        kaddr[s] + slot_bytes);
+    ka[1][s] = *reinterpret_cast<const __attribute__((address_space(3))) bf16x8*>(
+        kaddr[s] + slot_bytes + 16 * 256);
   }
 #pragma unroll
   for (int g = 0; g < kGroups; ++g) {
@@ -215,6 +257,10 @@ __device__ __forceinline__ void scores_of_tile(lds_ptr kt, const bf16x8 (&qreg)[
       sc[g][1] = Elem<F16>::mfma(ka[1][s], qreg[g][s], sc[g][1]);
     }
   }
+}
+__device__ __forceinline__ void k_read_addresses(lds_ptr k_lds, int r, int kg, lds_ptr (&kaddr)[4]) {
+#pragma unroll
+  for (int s = 0; s < 4; ++s) kaddr[s] = k_lds + 256 * r + 16 * k_position(r, 4 * s + kg);
 }
 
 // O^T += V^T . P^T and l += 1 . P^T for the probabilities `pb` of one tile whose
@@ -228,20 +274,20 @@ __device__ __forceinline__ void scores_of_tile(lds_ptr kt, const bf16x8 (&qreg)[
 // Every element of lacc[g] of a lane is the sum over all 32 keys of the tile for
 // the lane's query row: a ones-row times P^T on the matrix core, from the same
 // bf16 probabilities as the numerator.
+// vaddr[jd] is the lane's LDS address for operand jd in ring slot 0
+// (v_read_addresses); `slot_bytes` selects the ring slot.
 template <bool F16>
-__device__ __forceinline__ void accumulate_tile(lds_ptr vt, const bf16x8 (&pb)[kGroups],
-                                                f32x4 (&acc)[kGroups][8], f32x4 (&lacc)[kGroups], int r,
-                                                int kg) {
-  const int row = 4 * kg + (r >> 2);   // (16 + row) & 7 == row & 7: both reads share positions
-  const int chunk = r & 3;             // 8-byte chunk of the 32 bytes of a dimension group
+__device__ __forceinline__ void accumulate_tile(const lds_ptr (&vaddr)[8], int slot_bytes,
+                                                const bf16x8 (&pb)[kGroups],
+                                                f32x4 (&acc)[kGroups][8], f32x4 (&lacc)[kGroups]) {
   bf16x8 va[8];
 #pragma unroll
   for (int jd = 0; jd < 8; ++jd) {
-    const int at = 256 * row + 16 * v_position(row, 2 * jd + (chunk >> 1)) + 8 * (chunk & 1);
     const bf16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4bf16(
-        reinterpret_cast<__attribute__((address_space(3))) bf16x4*>(vt + at));
+        reinterpret_cast<__attribute__((address_space(3))) bf16x4*>(vaddr[jd] + slot_bytes));
     const bf16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4bf16(
-        reinterpret_cast<__attribute__((address_space(3))) bf16x4*>(vt + at + 16 * 256));
+        reinterpret_cast<__attribute__((address_space(3))) bf16x4*>(vaddr[jd] + slot_bytes +
+                                                                      16 * 256));
     va[jd] = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
   }
   const uint32_t one2 = Elem<F16>::kOnes;
@@ -253,6 +299,13 @@ __device__ __forceinline__ void accumulate_tile(lds_ptr vt, const bf16x8 (&pb)[k
     for (int jd = 0; jd < 8; ++jd)
       acc[g][jd] = Elem<F16>::mfma(va[jd], pb[g], acc[g][jd]);
   }
+}
+__device__ __forceinline__ void v_read_addresses(lds_ptr v_lds, int r, int kg, lds_ptr (&vaddr)[8]) {
+  const int row = 4 * kg + (r >> 2);   // (16 + row) & 7 == row & 7: both reads share positions
+  const int chunk = r & 3;             // 8-byte chunk of the 32 bytes of a dimension group
+#pragma unroll
+  for (int jd = 0; jd < 8; ++jd)
+    vaddr[jd] = v_lds + 256 * row + 16 * v_position(row, 2 * jd + (chunk >> 1)) + 8 * (chunk & 1);
 }
 
 // Probabilities of one tile from its scores (fp32 online softmax on the
@@ -468,53 +521,78 @@ __global__ __launch_bounds__(kWaves * 64, kGroups <= 2 ? 2 : 1) void prefill_att
   const int n_active = min(nsteps, (off + wave_row0 + kRowsPerWave - 1) / kKeys + 1);
   const int n_plain = min(min(off + wave_row0, k_end) / kKeys, n_active);
 
-  int k_stage = 0;   // ring slot of K of tile i
-  int v_stage = 0;   // ring slot of V of tile i (tile i-1 sits one slot before)
-#define NVJ_NEXT_TILE(i)                                                              \
-  do {                                                                                \
-    copier.issue((i) + 2, k_stage >= 1 ? k_stage - 1 : kKStages - 1,                  \
-                 v_stage >= 2 ? v_stage - 2 : v_stage + kVStages - 2);                \
-    wait_tiles_in_flight<1>();                                                        \
-    __syncthreads();                                                                  \
-    k_stage = k_stage + 1 == kKStages ? 0 : k_stage + 1;                              \
-    v_stage = v_stage + 1 == kVStages ? 0 : v_stage + 1;                              \
-  } while (0)
-#define NVJ_V_BEFORE() (v_lds + (v_stage >= 1 ? v_stage - 1 : kVStages - 1) * kTileBytes)
+  // Tile t lives in ring slot t % 4 (K and V alike).  Iteration i: scores of tile
+  // i, accumulation of tile i-1, probabilities of tile i, copies of tile i+2 into
+  // the slot last read in iteration i-1, wait for this lane's copies of tile i+1,
+  // barrier.
+  lds_ptr kaddr[4], vaddr[8];
+  k_read_addresses(k_lds, r, kg, kaddr);
+  v_read_addresses(v_lds, r, kg, vaddr);
+  uint32_t koff[kCopyRowsPerWave / 4], voff[kCopyRowsPerWave / 4];
+  copier.lane_offsets(koff, voff);
 
   f32x4 sc[kGroups][2];
   bf16x8 pb[kGroups];
 #pragma unroll
   for (int g = 0; g < kGroups; ++g) pb[g] = as_bf16x8(make_uint4(0u, 0u, 0u, 0u));
-  int i = 0;
   // Waves that issue matrix instructions go first: a wave lowers its priority
   // only while it turns scores into probabilities (vector ALU work that the
   // other wave of the SIMD can overlap with its own matrix instructions).
   __builtin_amdgcn_s_setprio(1);
-  for (; i < n_plain; ++i) {
-    scores_of_tile<F16>(k_lds + k_stage * kTileBytes, qreg, sc, r, kg);
-    accumulate_tile<F16>(NVJ_V_BEFORE(), pb, acc, lacc, r, kg);
-    __builtin_amdgcn_s_setprio(0);
-    probabilities_of_tile<false, F16>(sc, pb, acc, lacc, m_run, mneg, sl2, r, kg, 0, 0);
-    __builtin_amdgcn_s_setprio(1);
-    NVJ_NEXT_TILE(i);
+#define NVJ_END_OF_TILE()       \
+  do {                          \
+    wait_tiles_in_flight<1>();  \
+    __syncthreads();            \
+  } while (0)
+  // a plain tile whose ring slots are known when the code is written: every LDS
+  // offset is an immediate, the copies use the lanes' precomputed offsets
+#define NVJ_PLAIN_TILE_AT(S, i)                                                              \
+  do {                                                                                       \
+    scores_of_tile<F16>(kaddr, (S) * kTileBytes, qreg, sc);                                  \
+    accumulate_tile<F16>(vaddr, (((S) + 3) & 3) * kTileBytes, pb, acc, lacc);                \
+    __builtin_amdgcn_s_setprio(0);                                                           \
+    probabilities_of_tile<false, F16>(sc, pb, acc, lacc, m_run, mneg, sl2, r, kg, 0, 0);     \
+    __builtin_amdgcn_s_setprio(1);                                                           \
+    copier.template issue_full<((S) + 2) & 3>((i) + 2, koff, voff);                          \
+    NVJ_END_OF_TILE();                                                                       \
+  } while (0)
+  // any tile, ring slots computed at run time
+#define NVJ_TILE(MASKED, i, row_limit, key_limit)                                            \
+  do {                                                                                       \
+    scores_of_tile<F16>(kaddr, ((i) & 3) * kTileBytes, qreg, sc);                            \
+    accumulate_tile<F16>(vaddr, (((i) + 3) & 3) * kTileBytes, pb, acc, lacc);                \
+    __builtin_amdgcn_s_setprio(0);                                                           \
+    probabilities_of_tile<MASKED, F16>(sc, pb, acc, lacc, m_run, mneg, sl2, r, kg, row_limit, \
+                                       key_limit);                                           \
+    __builtin_amdgcn_s_setprio(1);                                                           \
+    copier.issue((i) + 2, ((i) + 2) & 3, ((i) + 2) & 3);                                     \
+    NVJ_END_OF_TILE();                                                                       \
+  } while (0)
+
+  int i = 0;
+  // four plain tiles at a time while the tiles they fetch (up to i + 5) are full ones
+  for (; i + 4 <= n_plain && i + 5 < nsteps - 1; i += 4) {
+    NVJ_PLAIN_TILE_AT(0, i);
+    NVJ_PLAIN_TILE_AT(1, i + 1);
+    NVJ_PLAIN_TILE_AT(2, i + 2);
+    NVJ_PLAIN_TILE_AT(3, i + 3);
   }
+  for (; i < n_plain; ++i) NVJ_TILE(false, i, 0, 0);
   for (; i < n_active; ++i) {
     const int ks = i * kKeys;
-    scores_of_tile<F16>(k_lds + k_stage * kTileBytes, qreg, sc, r, kg);
-    accumulate_tile<F16>(NVJ_V_BEFORE(), pb, acc, lacc, r, kg);
-    __builtin_amdgcn_s_setprio(0);
-    probabilities_of_tile<true, F16>(sc, pb, acc, lacc, m_run, mneg, sl2, r, kg, off + wave_row0 - ks,
-                                k_end - 1 - ks);
-    __builtin_amdgcn_s_setprio(1);
-    NVJ_NEXT_TILE(i);
+    NVJ_TILE(true, i, off + wave_row0 - ks, k_end - 1 - ks);
   }
   // the last tile of the wave is still to be accumulated; its V stays in place
   // until the copies of two iterations from now
-  if (n_active > 0) accumulate_tile<F16>(NVJ_V_BEFORE(), pb, acc, lacc, r, kg);
-  for (; i < nsteps; ++i) NVJ_NEXT_TILE(i);
+  if (n_active > 0) accumulate_tile<F16>(vaddr, ((i + 3) & 3) * kTileBytes, pb, acc, lacc);
+  for (; i < nsteps; ++i) {
+    copier.issue(i + 2, (i + 2) & 3, (i + 2) & 3);
+    NVJ_END_OF_TILE();
+  }
   wait_tiles_in_flight<0>();   // copies past the last tile are still landing in LDS
-#undef NVJ_NEXT_TILE
-#undef NVJ_V_BEFORE
+#undef NVJ_TILE
+#undef NVJ_PLAIN_TILE_AT
+#undef NVJ_END_OF_TILE
 
   // ---- epilogue: acc[g][jd][e] is O[row][dim = 16*jd + 4*kg + e] ----
 #pragma unroll
