@@ -57,7 +57,6 @@ constexpr int kTileBytes = kKeys * kD * 2;   // one K or V tile in LDS: 32 rows 
 // instruction immediate.
 constexpr int kKStages = 4;
 constexpr int kVStages = 4;
-constexpr int kStages = 4;
 constexpr float kNegBig = -1.0e30f;
 constexpr float kLazyLog2 = 8.0f;    // running max moves only for gains above 2^8
 constexpr float kLog2e = 1.4426950408889634f;
