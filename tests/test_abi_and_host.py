@@ -66,6 +66,19 @@ def test_argument_validation_without_a_gpu():
     assert P(None, x, x, x, x, x, x, x, 1 << 30, 2, 32, 8, 128, 256, 4, 16, 0.1, 0, 2, valu) == -3
     assert P(None, x, x, x, x, x, x, x, 1 << 30, 2, 32, 8, 128, 256, 4, 16, 0.1, 256, 0, valu) == -3
     assert P(None, x, x, x, x, x, x, x, 1 << 30, 0, 32, 8, 128, 256, 4, 16, 0.1, 0, 0, valu) == 0
+    # the loads-only measurement variant: head_dim 128, bf16, not with a fixed chunk or with valu
+    lo = _lib.NVJ_PHASE_SPLITK | _lib.NVJ_PHASE_LOADS_ONLY
+    assert P(None, x, x, x, x, x, x, x, 1 << 30, 2, 32, 8, 128, 256, 4, 16, 0.1, 256, 0, lo) == -3
+    assert P(None, x, x, x, x, x, x, x, 1 << 30, 2, 32, 8, 128, 256, 4, 16, 0.1, 0, 2, lo) == -3
+    assert P(None, x, x, x, x, x, x, x, 1 << 30, 2, 8, 2, 64, 256, 4, 16, 0.1, 0, 0, lo) == -3
+    assert P(None, x, x, x, x, x, x, x, 1 << 30, 2, 32, 8, 128, 256, 4, 16, 0.1, 0, 0,
+             lo | _lib.NVJ_PHASE_VALU_PRODUCTS) == -3
+    # counters of the balanced split: one int32 per (sequence, KV head as the kernels walk
+    # them: a group above 16 query heads counts as several), padded to 256 bytes
+    C = lib.nvj_paged_decode_counter_bytes
+    assert C(64, 32, 8) == 2048 and C(1, 8, 8) == 256 and C(3, 32, 1) == 256
+    assert C(100, 64, 2) == 1792          # 100 x (2 cache heads x 2 virtual heads of 16) x 4 B, padded
+    assert C(0, 32, 8) == 0 and C(4, 30, 8) == 0
     PP = lib.nvj_paged_prefill_attention_launch
     assert PP(None, x, x, x, x, x, x, x, 10, 2, 32, 8, 128, 48, 4, 16, 0.1, 0) == -3   # page % 32
     assert PP(None, x, x, x, x, x, x, x, 10, 2, 32, 8, 64, 64, 4, 16, 0.1, 0) == -3    # head_dim

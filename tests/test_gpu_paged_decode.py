@@ -604,3 +604,21 @@ def test_vector_alu_variant_refuses_other_shapes():
         kc = torch.zeros((2, 64, Hkv, D), dtype=dt, device=dev)
         with pytest.raises(_lib.NativeLibraryError, match="unsupported"):
             paged_attention(q, kc, kc, bt, ctx, 0.1, 64, chunk=chunk, phases=flags)
+
+
+def test_loads_only_variant_runs_and_leaves_finite_values():
+    """NVJ_PHASE_LOADS_ONLY (the K/V stream with no arithmetic behind it, a timing aid) runs
+    in both modes it exists for and leaves finite values in `out`."""
+    print("case loads-only variant", flush=True)
+    import torch
+    from nanovllm_jax_amd import _lib, paged_attention
+    B, Hq, Hkv, D, bs, NB = 7, 32, 8, 128, 64, 120
+    q, kc, vc, bt, ctx = make_problem(808, B, Hq, Hkv, D, bs, NB, [900, 33, 0, 640, 1, 1000, 257])
+    dev = "cuda:0"
+    for chunk in (0, -1):
+        out = paged_attention(bits_to_torch(q, dev), bits_to_torch(kc, dev), bits_to_torch(vc, dev),
+                              torch.from_numpy(bt).to(dev), torch.from_numpy(ctx).to(dev), 0.09, bs,
+                              chunk=chunk,
+                              phases=_lib.NVJ_PHASE_SPLITK | _lib.NVJ_PHASE_LOADS_ONLY)
+        torch.cuda.synchronize()
+        assert torch.isfinite(out.float()).all()
