@@ -622,3 +622,30 @@ def test_loads_only_variant_runs_and_leaves_finite_values():
                               phases=_lib.NVJ_PHASE_SPLITK | _lib.NVJ_PHASE_LOADS_ONLY)
         torch.cuda.synchronize()
         assert torch.isfinite(out.float()).all()
+
+
+@pytest.mark.parametrize("B,Hq,Hkv,bs,MB", [(64, 2, 1, 64, 8192),     # 1 KV head x 8 parts
+                                            (300, 8, 8, 32, 8192)])   # 8 KV heads x 1 part
+def test_balanced_split_with_a_very_wide_block_table(B, Hq, Hkv, bs, MB):
+    """The cut of the balanced split is computed in 32-bit arithmetic; when the block
+    table could describe so many positions that (steps x sub-runs) would not fit, the
+    kernel cuts in coarser units.  Only the table's width decides that, so short
+    sequences behind a table 8192 pages wide exercise it."""
+    print(f"case very wide block table B={B} Hkv={Hkv} MB={MB}", flush=True)
+    import torch
+    from nanovllm_jax_amd import paged_attention
+    rng = np.random.Generator(np.random.PCG64(B + MB))
+    D = 128
+    ctx = rng.integers(0, 900, size=B)
+    ctx[0] = 3000
+    q, kc, vc, bt, ctx = make_problem(5150 + B, B, Hq, Hkv, D, bs,
+                                      int((-(-ctx // bs)).sum()) + 1, ctx)
+    wide = np.full((B, MB), -1, np.int32)
+    wide[:, :bt.shape[1]] = bt
+    dev = "cuda:0"
+    out = paged_attention(bits_to_torch(q, dev), bits_to_torch(kc, dev), bits_to_torch(vc, dev),
+                          torch.from_numpy(wide).to(dev), torch.from_numpy(ctx).to(dev), 0.088, bs,
+                          chunk=0)
+    torch.cuda.synchronize()
+    assert_close_bf16(torch_to_bits(out), oracle(q, kc, vc, bt, ctx, 0.088, bs),
+                      what=f"wide table B={B}")
