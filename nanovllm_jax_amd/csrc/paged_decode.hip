@@ -903,8 +903,8 @@ __device__ __forceinline__ int wave_inclusive_scan(int x) {
 // ---------------------------------------------------------------------------
 // Balanced split: one launch for any mix of lengths.
 //
-// A workgroup is 8 waves = `hpw` KV heads x R = 8 / hpw parts (hpw is the
-// largest of 8, 4, 2, 1 that still leaves one row per CU, see the host side).
+// A workgroup is 8 waves = `hpw` KV heads x R = 8 / hpw parts (hpw is 4, 2 or
+// 1 by the size of the launch, see balanced_heads_per_workgroup on the host side).
 // The unit of work is a "row step": one 32-position step of one row, a row
 // being (sequence b, head group hg of hpw KV heads).  All row steps, ordered
 // by (b, hg, step), form one axis of length T = (num_kv_heads / hpw) * sum of
@@ -1157,7 +1157,7 @@ __device__ __forceinline__ void merge_row(const DecodeArgs& a, uint4* lds, int b
 template <int D, bool F16, int VG = 0>
 __global__ __launch_bounds__(512) void paged_decode_balanced_kernel(DecodeArgs a, int batch,
                                                                     int num_wgs, int min_steps,
-                                                                    int hpw, int shift,
+                                                                    int hpw, int alt_hpw, int shift,
                                                                     int32_t* counters) {
   using H = HeadDim<D>;
   constexpr int NW = 8;
@@ -1169,10 +1169,6 @@ __global__ __launch_bounds__(512) void paged_decode_balanced_kernel(DecodeArgs a
   const int lane = threadIdx.x & 63;
   const int g = blockIdx.x;
   const int cap = a.max_blocks * a.block_size;
-  const int parts = NW / hpw;
-  const int rows_per_seq = a.num_kv_heads / hpw;
-  const int part = wave / hpw;
-  const int h_in_row = wave - part * hpw;
 
   auto ctx_of = [&](int idx) { return idx < batch ? min(max(a.context_lens[idx], 0), cap) : 0; };
   auto steps_of = [&](int idx) { return (ctx_of(idx) + kStep - 1) / kStep; };
@@ -1185,6 +1181,8 @@ __global__ __launch_bounds__(512) void paged_decode_balanced_kernel(DecodeArgs a
 #pragma unroll
   for (int k = 0; k < kKeep; ++k) kept_ctx[k] = kept_excl[k] = 0;
   int total = 0, total_kept = 0;
+  const int steps0 = __builtin_amdgcn_readfirstlane(steps_of(0));
+  bool same_steps = true;   // every sequence has steps0 steps
 #pragma unroll
   for (int k = 0; k < kKeep; ++k) {
     if (k * 64 < batch) {
@@ -1193,13 +1191,26 @@ __global__ __launch_bounds__(512) void paged_decode_balanced_kernel(DecodeArgs a
       const int incl = wave_inclusive_scan(n);
       kept_excl[k] = total + incl - n;
       total += __builtin_amdgcn_readlane(incl, 63);
+      same_steps = same_steps && __ballot(k * 64 + lane < batch && n != steps0) == 0ull;
     }
   }
   total_kept = total;
   for (int base = kKeep * 64; base < batch; base += 64) {
     const int n = steps_of(base + lane);
     total += __builtin_amdgcn_readlane(wave_inclusive_scan(n), 63);
+    same_steps = same_steps && __ballot(base + lane < batch && n != steps0) == 0ull;
   }
+  // Sequences of one length whose rows of `alt_hpw` heads divide evenly over the
+  // workgroups: with that many heads per workgroup every run ends on a row
+  // boundary and no partial is ever written, which beats the better stream of
+  // `hpw` heads.  Every wave of the launch takes the same decision.
+  if (alt_hpw > 0 && same_steps &&
+      (int64_t)steps0 * (a.num_kv_heads / alt_hpw) * batch >= (int64_t)num_wgs * (NW / alt_hpw))
+    hpw = alt_hpw;
+  const int parts = NW / hpw;
+  const int rows_per_seq = a.num_kv_heads / hpw;
+  const int part = wave / hpw;
+  const int h_in_row = wave - part * hpw;
   // No step belongs to an empty sequence: its output row (zeros, 0 / (0 + 1e-9))
   // is written here, sequence b by workgroup b modulo the grid.  The lengths of
   // the first kKeep * 64 sequences are in registers already.
@@ -1493,14 +1504,34 @@ int compute_units() {
   return n;
 }
 
-// KV heads per 8-wave workgroup (whole-sequence and balanced modes): as many as
-// still give one (sequence, head group) row per CU, so that a sequence is split
-// over the waves of a workgroup no finer than needed; it must divide the number
-// of KV heads.
+// KV heads per 8-wave workgroup of the whole-sequence mode: as many as still
+// give one (sequence, head group) row per CU, so that a sequence is split over
+// the waves of a workgroup no finer than needed; it must divide the number of
+// KV heads.
 int heads_per_workgroup(int64_t batch, int num_kv_heads) {
   const int cus = compute_units();
   int hpw = 8;
   while (hpw > 1 && (num_kv_heads % hpw != 0 || batch * (num_kv_heads / hpw) < cus)) hpw /= 2;
+  return hpw;
+}
+
+// KV heads per 8-wave workgroup of the balanced split.  Two forces pull apart.
+// The heads of one workgroup read adjacent pieces of every position's row, and
+// a stream-bound launch runs faster with more of them side by side: 32
+// sequences of 16k..32k positions take 506 / 471 / 457 / 460 us with 1 / 2 / 4
+// / 8 heads of 128 per workgroup (head_dim 64 ranks the same way).  Against
+// that, the partials one wave has to merge per (sequence, head) grow with the
+// heads per workgroup, because the sub-runs are then spread over fewer rows: a
+// single sequence of 32k positions takes 38 / 45 / 67 / 109 us.  The rule below
+// is the best or within 3 % of it over batch 1..256 x 512..32768 positions x
+// 2, 4, 8 KV heads, ragged and uniform lengths: 4 heads from batch 32 up, or
+// from batch 16 when the table spans 4096 positions; 1 head for up to 16
+// (sequence, head) pairs when the table spans 6144 positions or more; else 2.
+int balanced_heads_per_workgroup(int64_t batch, int num_kv_heads, int64_t max_steps) {
+  int hpw = 2;
+  if (batch * num_kv_heads <= 16 && max_steps >= 192) hpw = 1;
+  else if (batch >= 32 || (batch >= 16 && max_steps >= 128)) hpw = 4;
+  while (hpw > 1 && num_kv_heads % hpw != 0) hpw /= 2;
   return hpw;
 }
 
@@ -1521,7 +1552,7 @@ int waves_per_workgroup(int num_kv_heads) {
 struct WorkspacePlan {
   int64_t records;  // partial records (one query head each)
   int max_chunks;   // fixed-chunk mode only
-  int num_wgs, hpw, shift; // balanced mode only
+  int num_wgs, hpw, alt_hpw, shift; // balanced mode only
   size_t counter_bytes;
   size_t bytes;
 };
@@ -1529,10 +1560,11 @@ struct WorkspacePlan {
 bool plan_workspace(int64_t batch, int64_t num_heads, int64_t head_dim, int64_t max_blocks,
                     int64_t block_size, int num_kv_heads, int chunk, WorkspacePlan* plan) {
   if (chunk == 0) {
-    const int hpw = heads_per_workgroup(batch, num_kv_heads);
+    const int64_t max_steps = (max_blocks * block_size + kStep - 1) / kStep;
+    const int hpw = balanced_heads_per_workgroup(batch, num_kv_heads, max_steps);
     const int parts = 8 / hpw;
     const int64_t rows_per_seq = num_kv_heads / hpw;
-    const int64_t axis = rows_per_seq * batch * ((max_blocks * block_size + kStep - 1) / kStep);
+    const int64_t axis = rows_per_seq * batch * max_steps;
     if (axis > INT32_MAX / 2) return false;
     int64_t wgs = (axis + (int64_t)parts * kMinBalancedSteps - 1) / (parts * kMinBalancedSteps);
     const int64_t cus = compute_units();
@@ -1542,6 +1574,15 @@ bool plan_workspace(int64_t batch, int64_t num_heads, int64_t head_dim, int64_t 
     // (units + 1) * sub-runs must fit 31 bits (Cut): coarser units for a very long axis
     plan->shift = 0;
     while ((((axis >> plan->shift) + 2) * wgs * parts) >> 31) ++plan->shift;
+    // Sequences of equal length need no partials at all when a workgroup's run is
+    // whole rows.  If 2 heads per workgroup give that and 4 do not, the kernel
+    // takes 2 when it finds the lengths equal (it reads them anyway).  Both
+    // layouts fill the same workspace: slots * hpw = 8 * workgroups + batch * heads.
+    plan->alt_hpw = 0;
+    const bool alt_fits_cut = plan->shift == 0 && (((2 * axis + 2) * wgs * 2 * parts) >> 31) == 0;
+    if (hpw == 4 && wgs == cus && alt_fits_cut && (batch * (num_kv_heads / 2)) % wgs == 0 &&
+        (batch * (num_kv_heads / 4)) % wgs != 0)
+      plan->alt_hpw = 2;
     plan->max_chunks = 0;
     const int64_t slots = wgs * parts + batch * rows_per_seq;
     plan->records = slots * hpw * (num_heads / num_kv_heads);
@@ -1551,7 +1592,7 @@ bool plan_workspace(int64_t batch, int64_t num_heads, int64_t head_dim, int64_t 
   }
   const int64_t mc = (max_blocks * block_size + chunk - 1) / chunk;
   if (batch * mc > INT32_MAX) return false;
-  plan->num_wgs = plan->hpw = plan->shift = 0;
+  plan->num_wgs = plan->hpw = plan->alt_hpw = plan->shift = 0;
   plan->max_chunks = (int)mc;
   plan->records = batch * mc * num_heads;
   plan->counter_bytes = 0;
@@ -1680,7 +1721,7 @@ int launch_decode(void* stream, const void* q, const void* k_cache, const void* 
     return rc == hipSuccess ? NVJ_OK : NVJ_ERR_LAUNCH;
   }
 
-  WorkspacePlan plan = {0, 1, 0, 0, 0, 0, 0};
+  WorkspacePlan plan = {0, 1, 0, 0, 0, 0, 0, 0};
   if (max_blocks > 0) {
     if (!plan_workspace(batch, num_heads, head_dim, max_blocks, block_size, num_kv_heads, chunk,
                         &plan))
@@ -1705,7 +1746,7 @@ int launch_decode(void* stream, const void* q, const void* k_cache, const void* 
       hipError_t rc;
 #define NVJ_LAUNCH_BALANCED(DV, F16V, VGV)                                                     \
   rc = nvj::launch(paged_decode_balanced_kernel<DV, F16V, VGV>, grid, dim3(512), s, a, batch, \
-                   plan.num_wgs, kMinBalancedSteps, plan.hpw, plan.shift, counters)
+                   plan.num_wgs, kMinBalancedSteps, plan.hpw, plan.alt_hpw, plan.shift, counters)
       if (loads_only) NVJ_LAUNCH_BALANCED(128, false, -1);
       else if (valu && group == 4) NVJ_LAUNCH_BALANCED(128, false, 4);
       else if (valu) NVJ_LAUNCH_BALANCED(128, false, 8);

@@ -105,10 +105,12 @@ def test_workspace_and_chunk_queries():
     # balanced split (no GPU here: 256 compute units assumed): counters, one int32 per
     # (sequence, KV head) padded to 256 bytes, then one partial slot per wave part of a
     # workgroup (<= 256 workgroups) plus one per (sequence, head group) row; at batch 64
-    # a workgroup is 2 KV heads x 4 parts, at batch 2 it is 1 KV head x 8 parts
+    # a workgroup is 4 KV heads x 2 parts, at batch 2 it is 2 KV heads x 4 parts, and 1 KV
+    # head x 8 parts for a single long sequence
     assert paged_decode_workspace_bytes(64, 32, 128, 16, 256, 8, 0) == \
-        2048 + (256 * 4 + 64 * 4) * 2 * 4 * (128 + 2) * 4
-    assert paged_decode_workspace_bytes(2, 8, 128, 1, 32, 8, 0) == 256 + (2 * 8 + 2 * 8) * 130 * 4
+        2048 + (256 * 2 + 64 * 2) * 4 * 4 * (128 + 2) * 4
+    assert paged_decode_workspace_bytes(2, 8, 128, 1, 32, 8, 0) == 256 + (2 * 4 + 2 * 4) * 2 * 130 * 4
+    assert paged_decode_workspace_bytes(1, 8, 128, 32, 256, 8, 0) == 256 + (256 * 8 + 8) * 130 * 4
 
 
 def test_host_mirror_refuses_cpu_tensors():

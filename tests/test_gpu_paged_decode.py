@@ -219,14 +219,18 @@ def test_balanced_split_many_ragged_sequences(B, seed):
 
 
 @pytest.mark.parametrize("B,Hq,Hkv,D,lo,hi", [
-    (3, 32, 8, 128, 0, 3000),      # 1 KV head x 8 parts per workgroup, rows over many workgroups
-    (64, 32, 8, 128, 0, 900),      # 2 x 4, runs cross rows of different head groups
-    (64, 16, 8, 128, 500, 512),    # 2 x 4, every row exactly one workgroup (no partials)
-    (130, 16, 8, 128, 0, 400),     # 4 x 2
-    (140, 8, 4, 64, 0, 300),       # head_dim 64, 2 x 4
+    (2, 32, 8, 128, 0, 3000),      # 1 KV head x 8 parts per workgroup, rows over many workgroups
+    (3, 32, 8, 128, 0, 3000),      # 2 x 4, rows over many workgroups
+    (10, 32, 8, 128, 0, 900),      # 2 x 4, runs cross rows of different head groups
+    (16, 16, 8, 128, 0, 1400),     # 4 x 2 because the table is wide
+    (64, 32, 8, 128, 0, 900),      # 4 x 2
+    (128, 16, 8, 128, 500, 512),   # 4 x 2, every row exactly one workgroup (no partials)
+    (64, 16, 8, 128, 500, 512),    # equal step counts: the kernel takes 2 x 4 instead, as above
+    (64, 16, 8, 128, 470, 512),    # 15 or 16 steps: stays 4 x 2, every row over two workgroups
+    (140, 8, 4, 64, 0, 300),       # head_dim 64, 4 x 2
     (90, 12, 6, 128, 0, 500),      # 6 KV heads: 2 per workgroup
     (40, 5, 5, 128, 0, 700),       # 5 KV heads: 1 per workgroup
-    (300, 8, 8, 128, 0, 200)])     # 8 x 1
+    (300, 8, 8, 128, 0, 200)])     # 4 x 2, more sequences than workgroups
 def test_balanced_split_every_workgroup_shape(B, Hq, Hkv, D, lo, hi):
     """chunk = 0 picks the KV heads per workgroup from the batch and head counts; every
     shape, with rows that are finished inside one workgroup, rows shared by parts of a
