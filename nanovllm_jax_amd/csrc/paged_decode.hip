@@ -1045,12 +1045,20 @@ __device__ __forceinline__ bool arrive(const DecodeArgs& a, int32_t* counters, i
   return true;
 }
 
+// x of the lane n places further on in its row of 16 lanes (wrapping around)
+template <int N>
+__device__ __forceinline__ float row_rotate(float x) {
+  return __builtin_bit_cast(
+      float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), 0x120 | N, 0xf, 0xf, false));
+}
+
 template <int D, bool F16>
 __device__ __forceinline__ void merge_row(const DecodeArgs& a, uint4* lds, int b, int kvh,
                                           int hpw, int r0, int r1, const Cut& cut, int lane) {
   using H = HeadDim<D>;
   // slots whose (max, sum) pairs fit the wave's tile at 16 heads x 8 bytes each
   constexpr int kSlots = (kStep * H::kLdsRowPieces * 16) / 128 >= 64 ? 64 : 32;
+  static_assert(kStep * H::kLdsRowPieces * 16 >= kSlots * 128 + kSlots, "room for the slot list");
   constexpr int KG = D / 32;
   const int parts = 8 / hpw;
   const int first = cut.subrun_of(r0);
@@ -1058,15 +1066,26 @@ __device__ __forceinline__ void merge_row(const DecodeArgs& a, uint4* lds, int b
   const int hg = kvh / hpw;
   const int rows_per_seq = a.num_kv_heads / hpw;
   const int64_t slot0 = (int64_t)first + (int64_t)b * rows_per_seq + hg;
-  // lanes of padding heads / padding dims read a real record and drop it later
-  const int r = min(lane & 15, a.group - 1);
+  // A row of 16 lanes has room for 16 query heads; with fewer, the row is cut
+  // into 16 / gp lane groups of gp >= group lanes (gp a power of two) and every
+  // lane group merges partials of its own, so that 4 * 16 / gp partials are in
+  // flight at once; the lane groups are added up at the end.  Lanes of padding
+  // heads / padding dims read a real record and drop it later.
+  const int gp = a.group > 8 ? 16 : a.group > 4 ? 8 : a.group > 2 ? 4 : a.group > 1 ? 2 : 1;
+  const int lane_groups = 16 / gp;
+  const int lg = (lane & 15) / gp;                        // this lane's group
+  const int r = min((lane & 15) - lg * gp, a.group - 1);  // its query head
   const int kg = (32 * (lane >> 4) < D) ? (lane >> 4) : 0;
   const int64_t rec0 = balanced_record(a, slot0, hpw, kvh - hg * hpw);   // slot0, head 0
   const int64_t rec_stride = (int64_t)hpw * a.group;                     // per slot
   const __amdgpu_buffer_rsrc_t wm = device_window(
       a.part_ml + rec0 * 2, ((int64_t)(expected - 1) * rec_stride + a.group) * 2 * sizeof(float));
+  const __amdgpu_buffer_rsrc_t wo = device_window(
+      a.part_o + rec0 * D, ((int64_t)(expected - 1) * rec_stride + a.group) * D * sizeof(float));
+  const int slot_bytes = (int)rec_stride * D * (int)sizeof(float);
   const int lane_off = (kg * a.group + r) * 16, piece_stride = KG * a.group * 16;
   vfloat2* lds_ml = reinterpret_cast<vfloat2*>(lds);   // [kSlots][16 heads]
+  uint8_t* lds_list = reinterpret_cast<uint8_t*>(lds_ml + kSlots * 16);   // [kSlots]
   f32x4 acc[8];
 #pragma unroll
   for (int jd = 0; jd < 8; ++jd) acc[jd] = f32x4{0.f, 0.f, 0.f, 0.f};
@@ -1081,53 +1100,56 @@ __device__ __forceinline__ void merge_row(const DecodeArgs& a, uint4* lds, int b
     const int g = j / parts;
     const bool inside = cut.start_of(g * parts) >= r0 &&
                         cut.start_of(min(cut.nsub, g * parts + parts)) <= r1;
-    unsigned long long real = __ballot(lane < count && (!inside || j == g * parts));
+    const bool mine_real = lane < count && (!inside || j == g * parts);
+    const unsigned long long real = __ballot(mine_real);
+    const int nreal = __popcll(real);
+    // the slots that hold a partial, in order, as a list
+    if (mine_real) lds_list[__popcll(real & ((1ull << lane) - 1ull))] = (uint8_t)lane;
     // (max, sum) of all these slots for the 16 head columns, the loads in flight
-    // together: lane (r, kg) fetches slot base + 4 * i + kg (unused slots hold
-    // stale values that are never looked at; slots past the end repeat the last).
+    // together: lane (column c, kg) fetches slot base + 4 * i + kg (unused slots
+    // hold stale values that are never looked at; slots past the end repeat the last).
     // (Fetching them together with the accumulators of the first partials, one
     // round trip fewer on paper, measured 2 us slower at 8 short sequences.)
+    const int c = min(lane & 15, a.group - 1);
     vfloat2 got[kSlots / 4];
 #pragma unroll
     for (int i = 0; i < kSlots / 4; ++i) {
       const int s = min(base + 4 * i + (lane >> 4), expected - 1);
       got[i] = __builtin_bit_cast(vfloat2, __builtin_amdgcn_raw_buffer_load_b64(
-                                               wm, (int)((s * rec_stride + r) * 8), 0, kDeviceScope));
+                                               wm, (int)((s * rec_stride + c) * 8), 0, kDeviceScope));
     }
 #pragma unroll
     for (int i = 0; i < kSlots / 4; ++i) lds_ml[(4 * i + (lane >> 4)) * 16 + (lane & 15)] = got[i];
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
     __builtin_amdgcn_wave_barrier();
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-    if (real != 0ull) {
+    if (nreal > 0) {
       float m_chunk = kNegBig;
       for (unsigned long long todo = real; todo != 0ull; todo &= todo - 1ull)
-        m_chunk = fmaxf(m_chunk, lds_ml[__builtin_ctzll(todo) * 16 + (lane & 15)].x);
+        m_chunk = fmaxf(m_chunk, lds_ml[__builtin_ctzll(todo) * 16 + r].x);
       const float m_new = fmaxf(m_run, m_chunk);
       const float keep = __builtin_amdgcn_exp2f((m_run - m_new) * a.scale_log2e);
       m_run = m_new;
       l_run *= keep;
 #pragma unroll
       for (int jd = 0; jd < 8; ++jd) acc[jd] *= keep;
-      while (real != 0ull) {
-        // up to four partials at a time; absent ones repeat the first with weight 0
-        int idx[4];
+      for (int done = 0; done < nreal; done += 4 * lane_groups) {
+        // four partials per lane group at a time; absent ones repeat the first
+        // of the list with weight 0
         float w[4];
         vfloat4 v[4][8];
 #pragma unroll
         for (int k = 0; k < 4; ++k) {
-          const bool have = real != 0ull;
-          idx[k] = have ? __builtin_ctzll(real) : idx[0];
-          if (have) real &= real - 1ull;
-          const __amdgpu_buffer_rsrc_t win =
-              device_window(a.part_o + (rec0 + (base + idx[k]) * rec_stride) * D,
-                            (int64_t)a.group * D * sizeof(float));
+          const int n = done + k * lane_groups + lg;
+          const bool have = n < nreal;
+          const int idx = lds_list[have ? n : 0];
+          const int off = (base + idx) * slot_bytes + lane_off;
 #pragma unroll
           for (int i = 0; i < 8; ++i)
             v[k][i] = __builtin_bit_cast(
-                vfloat4, __builtin_amdgcn_raw_buffer_load_b128(win, lane_off + i * piece_stride, 0,
-                                                               kDeviceScope));
-          const vfloat2 ml = lds_ml[idx[k] * 16 + (lane & 15)];
+                vfloat4,
+                __builtin_amdgcn_raw_buffer_load_b128(wo, off + i * piece_stride, 0, kDeviceScope));
+          const vfloat2 ml = lds_ml[idx * 16 + r];
           w[k] = have ? __builtin_amdgcn_exp2f((ml.x - m_new) * a.scale_log2e) : 0.f;
           l_run = fmaf(w[k], ml.y, l_run);
         }
@@ -1147,8 +1169,21 @@ __device__ __forceinline__ void merge_row(const DecodeArgs& a, uint4* lds, int b
       }
     }
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-    __builtin_amdgcn_wave_barrier();   // the next pass overwrites lds_ml
+    __builtin_amdgcn_wave_barrier();   // the next pass overwrites lds_ml and the list
   }
+  // the sum over the lane groups, into every lane
+#define NVJ_ADD_LANE_GROUPS(N)                                         \
+  if (gp <= N) {                                                       \
+    l_run += row_rotate<N>(l_run);                                     \
+    _Pragma("unroll") for (int jd = 0; jd < 8; ++jd)                   \
+      _Pragma("unroll") for (int e = 0; e < 4; ++e)                    \
+        acc[jd][e] += row_rotate<N>(acc[jd][e]);                       \
+  }
+  NVJ_ADD_LANE_GROUPS(8)
+  NVJ_ADD_LANE_GROUPS(4)
+  NVJ_ADD_LANE_GROUPS(2)
+  NVJ_ADD_LANE_GROUPS(1)
+#undef NVJ_ADD_LANE_GROUPS
   write_output<D, F16>(a, b, kvh, lane, acc, l_run);
 }
 
