@@ -1139,9 +1139,17 @@ __device__ __forceinline__ void merge_row(const DecodeArgs& a, uint4* lds, int b
     __builtin_amdgcn_wave_barrier();
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
     if (nreal > 0) {
+      // the largest maximum among the real slots, per head: over the slots this
+      // lane fetched, over the four lane rows, then from the head's column
       float m_chunk = kNegBig;
-      for (unsigned long long todo = real; todo != 0ull; todo &= todo - 1ull)
-        m_chunk = fmaxf(m_chunk, lds_ml[__builtin_ctzll(todo) * 16 + r].x);
+#pragma unroll
+      for (int i = 0; i < kSlots / 4; ++i) {
+        const int sl = min(4 * i + (lane >> 4), count - 1);
+        if ((real >> sl) & 1ull) m_chunk = fmaxf(m_chunk, got[i].x);
+      }
+      m_chunk = fmaxf(m_chunk, __shfl_xor(m_chunk, 16, 64));
+      m_chunk = fmaxf(m_chunk, __shfl_xor(m_chunk, 32, 64));
+      m_chunk = __shfl(m_chunk, (lane & 48) | r, 64);
       const float m_new = fmaxf(m_run, m_chunk);
       const float keep = __builtin_amdgcn_exp2f((m_run - m_new) * a.scale_log2e);
       m_run = m_new;
