@@ -227,6 +227,8 @@ def test_balanced_split_many_ragged_sequences(B, seed):
     (128, 16, 8, 128, 500, 512),   # 4 x 2, every row exactly one workgroup (no partials)
     (64, 16, 8, 128, 500, 512),    # equal step counts: the kernel takes 2 x 4 instead, as above
     (64, 16, 8, 128, 470, 512),    # 15 or 16 steps: stays 4 x 2, every row over two workgroups
+    (64, 8, 8, 64, 250, 256),      # head_dim 64, equal step counts: 2 x 4 taken on the device
+    (128, 8, 4, 128, 500, 512),    # 4 KV heads, equal step counts: 128 rows of 4, 256 of 2 -> 2 x 4
     (140, 8, 4, 64, 0, 300),       # head_dim 64, 4 x 2
     (90, 12, 6, 128, 0, 500),      # 6 KV heads: 2 per workgroup
     (40, 5, 5, 128, 0, 700),       # 5 KV heads: 1 per workgroup
