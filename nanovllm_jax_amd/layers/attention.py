@@ -41,6 +41,11 @@ def _raw_stream(device_index: int) -> int:
         return torch.cuda.current_stream(device_index).cuda_stream
 
 
+# the current device without the bookkeeping of torch.cuda.current_device()
+_current_device = getattr(torch._C, "_cuda_getDevice", None) or torch.cuda.current_device
+_store_launch = None    # the library's entry point, looked up at the first call
+
+
 # What a call signature (shapes, dtypes, devices of the five tensors) was validated
 # to: the integer arguments of the launch.  Validation is by far the larger part of
 # an eager call of this 3-microsecond kernel, so it runs once per signature.
@@ -105,17 +110,19 @@ def store_kv_to_cache(key, value, k_cache, v_cache, slot_mapping):
             and v_cache.is_contiguous() and slot_mapping.is_contiguous()):
         raise ValueError("key, value, k_cache, v_cache and slot_mapping must be contiguous")
     dev, num_tokens, num_kv_heads, head_dim, num_slots, kd, vd, cd = plan
-    if torch.cuda.current_device() == dev:
-        code = _lib.load().nvj_store_kvcache_launch(
-            _raw_stream(dev), key.data_ptr(), value.data_ptr(), k_cache.data_ptr(),
-            v_cache.data_ptr(), slot_mapping.data_ptr(), num_tokens, num_kv_heads, head_dim,
-            num_slots, kd, vd, cd)
+    global _store_launch
+    launch = _store_launch
+    if launch is None:
+        launch = _store_launch = _lib.load().nvj_store_kvcache_launch
+    if _current_device() == dev:
+        code = launch(_raw_stream(dev), key.data_ptr(), value.data_ptr(), k_cache.data_ptr(),
+                      v_cache.data_ptr(), slot_mapping.data_ptr(), num_tokens, num_kv_heads,
+                      head_dim, num_slots, kd, vd, cd)
     else:
         with torch.cuda.device(dev):
-            code = _lib.load().nvj_store_kvcache_launch(
-                _raw_stream(dev), key.data_ptr(), value.data_ptr(), k_cache.data_ptr(),
-                v_cache.data_ptr(), slot_mapping.data_ptr(), num_tokens, num_kv_heads, head_dim,
-                num_slots, kd, vd, cd)
+            code = launch(_raw_stream(dev), key.data_ptr(), value.data_ptr(), k_cache.data_ptr(),
+                          v_cache.data_ptr(), slot_mapping.data_ptr(), num_tokens, num_kv_heads,
+                          head_dim, num_slots, kd, vd, cd)
     if code != 0:
         _lib.check(code, "nvj_store_kvcache_launch")
     return k_cache, v_cache
