@@ -254,6 +254,28 @@ def test_balanced_split_every_workgroup_shape(B, Hq, Hkv, D, lo, hi):
     assert not got[ctx == 0].any()
 
 
+@pytest.mark.parametrize("odd_one", [None, 3, 300])
+def test_balanced_split_layout_chosen_on_the_device(odd_one):
+    """384 sequences x 4 KV heads of 8 steps each: the host plans 4 KV heads per
+    workgroup (384 rows over 256 workgroups), the kernel finds the step counts
+    equal and takes 2 KV heads (768 rows, 3 whole rows per workgroup, no partials).
+    One shorter sequence, among the first 256 whose lengths a wave keeps or
+    beyond them, and it must stay with the host's plan.  Both against the oracle."""
+    print(f"case device-chosen layout odd_one={odd_one}", flush=True)
+    B, Hq, Hkv, D, bs = 384, 8, 4, 128, 64
+    rng = np.random.Generator(np.random.PCG64(77))
+    ctx = rng.integers(250, 257, size=B)        # 8 steps of 32 each
+    if odd_one is not None:
+        ctx[odd_one] = 100                      # 4 steps
+    NB = int((-(-ctx // bs)).sum()) + 2
+    q, kc, vc, bt, ctx = make_problem(4242, B, Hq, Hkv, D, bs, NB, ctx)
+    scale = 1.0 / np.sqrt(D)
+    got = run_hip(q, kc, vc, bt, ctx, scale, bs, 0)
+    want = oracle(q, kc, vc, bt, ctx, scale, bs)
+    assert_close_bf16(got, want, what=f"device-chosen layout odd_one={odd_one}")
+
+
+
 @pytest.mark.parametrize("B,Hkv", [(6, 8), (64, 8), (300, 4)])
 def test_balanced_split_is_one_launch_that_leaves_its_counters_zero(B, Hkv):
     """With a DecodeWorkspace (counters zero from the start) a chunk = 0 call is a single
