@@ -947,6 +947,10 @@ __device__ __forceinline__ int wave_inclusive_scan(int x) {
 // puts the counter back to zero.  Nothing ever waits for another workgroup.
 // ---------------------------------------------------------------------------
 
+// Sequences whose (length, steps before) pairs every wave keeps in registers
+// after its one pass over the lengths; further ones are read again when needed.
+constexpr int kKeptSequences = 256;
+
 // The cut of the axis: sub-run j covers the axis positions whose unit
 // (position >> shift) lies in [floor(j * units / nsub), floor((j+1) * units / nsub)).
 // shift is 0 unless the axis is so long that units * nsub would not fit 31 bits
@@ -1234,7 +1238,7 @@ __global__ __launch_bounds__(512) void paged_decode_balanced_kernel(DecodeArgs a
   // One pass over the batch, 64 sequences at a time: total number of steps,
   // and for the first kKeep groups the per-lane (length, steps before) pairs
   // are kept so that locating a position below needs no second read.
-  constexpr int kKeep = 4;
+  constexpr int kKeep = kKeptSequences / 64;
   int kept_ctx[kKeep], kept_excl[kKeep];
 #pragma unroll
   for (int k = 0; k < kKeep; ++k) kept_ctx[k] = kept_excl[k] = 0;
@@ -1256,15 +1260,14 @@ __global__ __launch_bounds__(512) void paged_decode_balanced_kernel(DecodeArgs a
   for (int base = kKeep * 64; base < batch; base += 64) {
     const int n = steps_of(base + lane);
     total += __builtin_amdgcn_readlane(wave_inclusive_scan(n), 63);
-    same_steps = same_steps && __ballot(base + lane < batch && n != steps0) == 0ull;
   }
-  // Sequences of one length whose rows of `alt_hpw` heads divide evenly over the
-  // workgroups: with that many heads per workgroup every run ends on a row
-  // boundary and no partial is ever written, which beats the better stream of
-  // `hpw` heads.  Every wave of the launch takes the same decision.
-  if (alt_hpw > 0 && same_steps &&
-      (int64_t)steps0 * (a.num_kv_heads / alt_hpw) * batch >= (int64_t)num_wgs * (NW / alt_hpw))
-    hpw = alt_hpw;
+  // Sequences of one length and exactly one row of `alt_hpw` heads per workgroup
+  // (the host offers alt_hpw only then, and only for a batch whose lengths are
+  // all among the kept ones): with that many heads per workgroup every run is
+  // one whole row, its parts meet in LDS and no partial is ever written, which
+  // beats the better stream of `hpw` heads.  Every wave of the launch takes
+  // the same decision.
+  if (alt_hpw > 0 && same_steps && steps0 >= NW / alt_hpw) hpw = alt_hpw;
   const int parts = NW / hpw;
   const int rows_per_seq = a.num_kv_heads / hpw;
   const int part = wave / hpw;
@@ -1623,14 +1626,15 @@ bool plan_workspace(int64_t batch, int64_t num_heads, int64_t head_dim, int64_t 
     // (units + 1) * sub-runs must fit 31 bits (Cut): coarser units for a very long axis
     plan->shift = 0;
     while ((((axis >> plan->shift) + 2) * wgs * parts) >> 31) ++plan->shift;
-    // Sequences of equal length need no partials at all when a workgroup's run is
-    // whole rows.  If 2 heads per workgroup give that and 4 do not, the kernel
-    // takes 2 when it finds the lengths equal (it reads them anyway).  Both
-    // layouts fill the same workspace: slots * hpw = 8 * workgroups + batch * heads.
+    // Sequences of equal length need no partials at all when every workgroup's
+    // run is exactly one row.  If 2 heads per workgroup give that (and 4 would
+    // share every row between two workgroups), the kernel takes 2 when it finds
+    // the lengths equal (it reads them anyway).  Both layouts fill the same
+    // workspace: slots * hpw = 8 * workgroups + batch * heads.
     plan->alt_hpw = 0;
     const bool alt_fits_cut = plan->shift == 0 && (((2 * axis + 2) * wgs * 2 * parts) >> 31) == 0;
-    if (hpw == 4 && wgs == cus && alt_fits_cut && (batch * (num_kv_heads / 2)) % wgs == 0 &&
-        (batch * (num_kv_heads / 4)) % wgs != 0)
+    if (hpw == 4 && wgs == cus && alt_fits_cut && batch * (num_kv_heads / 2) == wgs &&
+        batch <= kKeptSequences)
       plan->alt_hpw = 2;
     plan->max_chunks = 0;
     const int64_t slots = wgs * parts + batch * rows_per_seq;

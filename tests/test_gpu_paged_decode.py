@@ -254,15 +254,16 @@ def test_balanced_split_every_workgroup_shape(B, Hq, Hkv, D, lo, hi):
     assert not got[ctx == 0].any()
 
 
-@pytest.mark.parametrize("odd_one", [None, 3, 300])
+@pytest.mark.parametrize("odd_one", [None, 3, 100])
 def test_balanced_split_layout_chosen_on_the_device(odd_one):
-    """384 sequences x 4 KV heads of 8 steps each: the host plans 4 KV heads per
-    workgroup (384 rows over 256 workgroups), the kernel finds the step counts
-    equal and takes 2 KV heads (768 rows, 3 whole rows per workgroup, no partials).
-    One shorter sequence, among the first 256 whose lengths a wave keeps or
-    beyond them, and it must stay with the host's plan.  Both against the oracle."""
+    """128 sequences x 4 KV heads of 8 steps each: the host plans 4 KV heads per
+    workgroup (128 rows, each shared by two of the 256 workgroups); the kernel finds
+    the step counts equal and takes 2 KV heads instead (256 rows, one whole row per
+    workgroup, merged in LDS): nothing is written to the workspace.  With one
+    shorter sequence it must stay with the host's plan, and partials appear.  Both
+    against the oracle."""
     print(f"case device-chosen layout odd_one={odd_one}", flush=True)
-    B, Hq, Hkv, D, bs = 384, 8, 4, 128, 64
+    B, Hq, Hkv, D, bs = 128, 8, 4, 128, 64
     rng = np.random.Generator(np.random.PCG64(77))
     ctx = rng.integers(250, 257, size=B)        # 8 steps of 32 each
     if odd_one is not None:
@@ -270,9 +271,24 @@ def test_balanced_split_layout_chosen_on_the_device(odd_one):
     NB = int((-(-ctx // bs)).sum()) + 2
     q, kc, vc, bt, ctx = make_problem(4242, B, Hq, Hkv, D, bs, NB, ctx)
     scale = 1.0 / np.sqrt(D)
-    got = run_hip(q, kc, vc, bt, ctx, scale, bs, 0)
+    import torch
+    from nanovllm_jax_amd import _lib, paged_attention
+    from nanovllm_jax_amd.layers.paged_attention import paged_decode_workspace_bytes
+    dev = "cuda:0"
+    # a workspace full of ones: whatever is still all ones afterwards was not written
+    ws = torch.full((paged_decode_workspace_bytes(B, Hq, D, bt.shape[1], bs, Hkv, 0),), 0xFF,
+                    dtype=torch.uint8, device=dev)
+    out = paged_attention(bits_to_torch(q, dev), bits_to_torch(kc, dev), bits_to_torch(vc, dev),
+                          torch.from_numpy(bt).to(dev), torch.from_numpy(ctx).to(dev), scale, bs,
+                          chunk=0, workspace=ws)
+    torch.cuda.synchronize()
     want = oracle(q, kc, vc, bt, ctx, scale, bs)
-    assert_close_bf16(got, want, what=f"device-chosen layout odd_one={odd_one}")
+    assert_close_bf16(torch_to_bits(out), want, what=f"device-chosen layout odd_one={odd_one}")
+    counters = int(_lib.load().nvj_paged_decode_counter_bytes(B, Hq, Hkv))
+    assert not ws[:counters].any(), "counters are zero after the call"
+    partials_untouched = bool((ws[counters:] == 0xFF).all())
+    assert partials_untouched == (odd_one is None), \
+        "equal step counts: no partial is written; one odd sequence: some are"
 
 
 
