@@ -943,8 +943,9 @@ __device__ __forceinline__ int wave_inclusive_scan(int x) {
 // head), zero between launches.  A wave that has written partials for a row
 // adds the number of sub-runs they stand for; the wave whose addition
 // completes the row's count (the number of sub-runs that touch the row, known
-// from the cut) merges the row's partials in slot order, writes the output and
-// puts the counter back to zero.  Nothing ever waits for another workgroup.
+// from the cut) merges the row's partials (in an order fixed by the cut alone,
+// so that the result does not depend on who merges), writes the output and puts
+// the counter back to zero.  Nothing ever waits for another workgroup.
 // ---------------------------------------------------------------------------
 
 // Sequences whose (length, steps before) pairs every wave keeps in registers
@@ -1037,8 +1038,8 @@ __device__ __forceinline__ void wait_for_stores() {
 
 // arrive: the wave has written its partials of row [r0, r1) (row steps on the
 // axis) of (sequence b, KV head kvh), standing for `n` sub-runs, and publishes
-// them.  merge_row: all partials of the row are there; merge them in slot order
-// and write the output.  `lds` is the wave's own tile (free at that point).
+// them.  merge_row: all partials of the row are there; merge them and write the
+// output.  `lds` is the wave's own tile (free at that point).
 //
 // The merge keeps the chain of dependent memory round trips short: which slots
 // hold a partial is computed from the cut, not read; the (max, sum) pairs of up
