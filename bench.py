@@ -296,7 +296,7 @@ def prefill_record(lens, prefix, steps, warmup, torch):
 
 
 def decode_record(name, chunk, dtype, products, steps, warmup, torch, dev, in_graph=False,
-                  keep_inputs=False, warm_seconds=0.0):
+                  keep_inputs=False, warm_seconds=0.0, shared_rows=False):
     """Time the decode call (and the KV store) on one workload.  Returns the
     measurements, plus the device inputs when `keep_inputs`.  `warm_seconds`:
     keep making untimed calls for that long after the `warmup` calls (a workload
@@ -316,6 +316,8 @@ def decode_record(name, chunk, dtype, products, steps, warmup, torch, dev, in_gr
     vflat = vc.view(-1, w.num_kv_heads, w.head_dim)
     variant = {"valu": _lib.NVJ_PHASE_VALU_PRODUCTS, "none": _lib.NVJ_PHASE_LOADS_ONLY}.get(
         products, 0)
+    if shared_rows:      # the equal cut with rows shared between workgroups, whatever the lengths
+        variant |= _lib.NVJ_PHASE_SHARED_ROWS
 
     def decode(phases=_lib.NVJ_PHASE_SPLITK | _lib.NVJ_PHASE_COMBINE):
         paged_attention(q, kc, vc, bt, ctx, w.scale, w.block_size, chunk=chunk, out=out,
@@ -384,6 +386,17 @@ def others_block(args, torch, dev):
     warm = dict(warm_seconds=0.2)
     run("C2_whole_sequence_split", lambda: brief(decode_record("C2", -1, "bf16", "mfma", st, wu,
                                                               torch, dev, **warm)))
+    # the headline batch is the special case of equal lengths (whole rows dealt to the
+    # workgroups, nothing shared): the same shape with lengths that differ, and with
+    # the general layout (rows shared between workgroups) forced
+    run("C2_jitter_ctx_3840_4096", lambda: brief(decode_record(
+        "C2_JITTER", 0, "bf16", "mfma", st, wu, torch, dev, **warm)))
+    run("C2_spread_ctx_2048_6144", lambda: brief(decode_record(
+        "C2_SPREAD", 0, "bf16", "mfma", st, wu, torch, dev, **warm)))
+    run("C2_rows_shared_between_workgroups", lambda: brief(decode_record(
+        "C2", 0, "bf16", "mfma", st, wu, torch, dev, shared_rows=True, **warm)))
+    run("ragged_short_B256_ctx_200_2048", lambda: brief(decode_record(
+        "RAGGED_SHORT", 0, "bf16", "mfma", st, wu, torch, dev, **warm)))
     run("C1", lambda: brief(decode_record("C1", 0, "bf16", "mfma", st, wu, torch, dev,
                                           in_graph=True, **warm)))
     run("C5_layer", lambda: brief(decode_record("C5", 0, "bf16", "mfma", st, wu, torch, dev,
@@ -412,7 +425,12 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
-    ap.add_argument("--workload", default="C2", choices=["C1", "C2", "C3", "C4", "C5", "R1"])
+    ap.add_argument("--workload", default="C2",
+                    choices=["C1", "C2", "C3", "C4", "C5", "R1", "C2_JITTER", "C2_SPREAD",
+                             "RAGGED_SHORT"])
+    ap.add_argument("--shared-rows", action="store_true",
+                    help="balanced split: keep the kernel from dealing whole rows to the "
+                         "workgroups (the equal cut with shared rows, whatever the lengths)")
     ap.add_argument("--chunk", type=int, default=0,
                     help="split mode: 0 = balanced (one launch, the default), > 0 = positions "
                          "per workgroup plus a combine launch, -1 = whole sequence per workgroup")
@@ -477,7 +495,8 @@ def main():
     # the W warm-up calls are 3 ms of work; the clocks of an idle GPU take longer to
     # come up, so untimed calls go on for a fifth of a second before the K timed ones
     m = decode_record(args.workload, chunk, args.dtype, args.products, args.steps, args.warmup,
-                      torch, dev, in_graph=True, keep_inputs=True, warm_seconds=0.2)
+                      torch, dev, in_graph=True, keep_inputs=True, warm_seconds=0.2,
+                      shared_rows=args.shared_rows)
     w = m["workload"]
     split_name = {0: "balanced", -1: "whole sequence per workgroup"}.get(chunk,
                                                                         f"fixed chunk {chunk}")
@@ -501,7 +520,9 @@ def main():
                                f"D={w.head_dim} page={w.block_size} "
                                f"ctx={int(w.context_lens.min())}..{int(w.context_lens.max())} "
                                f"pool={w.num_blocks} pages",
-                   "split": split_name, "products": args.products,
+                   "split": split_name + (", rows shared between workgroups forced"
+                                          if args.shared_rows else ""),
+                   "products": args.products,
                    "algorithmic_bytes_per_call": byts,
                    "step": "split-K launch + combine launch" if chunk > 0 else "one launch"},
         "roofline": {"bound": "hbm", "achieved": round(gbps_kernel, 1), "peak": HBM_PEAK_GBPS,

@@ -26,7 +26,7 @@
 extern "C" {
 #endif
 
-#define NVJ_ABI_VERSION 2
+#define NVJ_ABI_VERSION 3
 
 /* exported from the shared library (which is built with hidden visibility) */
 #define NVJ_API __attribute__((visibility("default")))
@@ -90,14 +90,19 @@ NVJ_API int nvj_store_kvcache_launch(void* stream,
  * How the positions of a call are split over workgroups is chosen by `chunk`:
  *
  *   chunk == 0  balanced split (the default), ONE launch for any mix of
- *               lengths: the 32-position steps of all (sequence, head group)
- *               rows, end to end, are cut into equal runs, one per wave, at
- *               most one 8-wave workgroup per CU.  The kernel derives the cut
- *               from context_lens on the device, so ragged batches are
- *               balanced without the host knowing the lengths; a row that
- *               fits one workgroup is finished there, a row shared by several
- *               is merged by the wave that completes it (counters in the
- *               workspace), without a second launch.
+ *               lengths, at most one 8-wave workgroup per CU.  The kernel reads
+ *               context_lens on the device and lays the work out itself, so
+ *               ragged batches are balanced without the host knowing the
+ *               lengths.  Where whole (sequence, head group) rows can be dealt
+ *               to the workgroups within 1/16 of an equal share of the
+ *               32-position steps (lengths equal or nearly so; or, taken by
+ *               decreasing length, long rows that pair up with short ones), no
+ *               row is shared between workgroups and the workspace is not
+ *               touched.  Otherwise the steps of all rows, end to end, are cut
+ *               into equal runs, one per wave; a row that fits one workgroup is
+ *               finished there, a row shared by several is merged by the wave
+ *               that completes it (counters in the workspace), without a
+ *               second launch.
  *   chunk  > 0  fixed split: workgroup (b, c) takes positions
  *               [c * chunk, (c + 1) * chunk) of sequence b; chunk must be a
  *               multiple of 32.
@@ -137,10 +142,11 @@ NVJ_API int32_t nvj_paged_decode_whole_sequence_workgroups(int32_t batch, int32_
  * balanced size depends on the number of compute units of the current device.
  *
  * nvj_paged_decode_counter_bytes: how many bytes at the head of a balanced-split
- * workspace are its counters (one int32 per (sequence, KV head), padded to 256
- * bytes; 0 on invalid arguments).  A caller that reuses one workspace for
- * calls of different shapes needs it: a launch leaves exactly that prefix zero,
- * what lies behind it holds partials.
+ * workspace are its counter region (int32 words: word 0 is the stale flag
+ * described at nvj_paged_decode_launch_phases, then one counter per (sequence,
+ * KV head); padded to 256 bytes; 0 on invalid arguments).  What lies behind it
+ * holds partials; nvj_paged_decode_launch_counters takes the two as separate
+ * buffers.
  */
 NVJ_API size_t nvj_paged_decode_counter_bytes(int32_t batch, int32_t num_heads,
                                              int32_t num_kv_heads);
@@ -202,14 +208,25 @@ NVJ_API int nvj_paged_decode_launch(void* stream,
  * > 0 the partials stay in `workspace`).  NVJ_PHASE_COMBINE: the second pass of
  * the fixed split (reads the partials an earlier split-K launch with the same
  * arguments left in `workspace`; nothing for the other modes).
- * NVJ_PHASE_CLEAR_COUNTERS: chunk == 0 only, set the counters at the head of
- * `workspace` to zero first.  The balanced kernel needs them zero when it
- * starts and leaves them zero when it ends, so a caller that keeps one
+ * NVJ_PHASE_CLEAR_COUNTERS: chunk == 0 only, set the counter region at the head
+ * of `workspace` to zero first.  The balanced kernel needs the counters zero
+ * when it starts and leaves them zero when it ends, so a caller that keeps one
  * workspace per stream clears it once (this bit alone, or with the first call)
- * and then passes NVJ_PHASE_SPLITK only: one launch per call.  A workspace whose
- * counters are not zero gives wrong results (never a fault).  All three bits =
+ * and then passes NVJ_PHASE_SPLITK only: one launch per call.  Calls of
+ * different shapes must not share such a workspace (the counter region of one
+ * shape overlaps the partials of another; nvj_paged_decode_launch_counters keeps
+ * the two apart).  A counter that was not zero is noticed by the wave that finds
+ * more arrivals than the row has pieces: it sets word 0 of the counter region
+ * (the stale flag; sticky until the region is cleared) to 1, puts the counter
+ * back to zero and leaves that row of `out` unwritten.  Every kernel still ends
+ * normally (never a fault, never a wait); a caller that cannot rule the
+ * condition out reads the flag back after the call.  All three bits =
  * nvj_paged_decode_launch.  Same reference counterpart as
  * nvj_paged_decode_launch.
+ *
+ * NVJ_PHASE_SHARED_ROWS, or-ed in, keeps the balanced split from dealing whole
+ * rows (see chunk == 0 above): the equal cut with shared rows is taken whatever
+ * the lengths.  Same results to the same tolerance; a measurement and test aid.
  *
  * NVJ_PHASE_VALU_PRODUCTS, or-ed in, runs a measurement variant of the split-K
  * kernel that computes Q.K and P.V with vector-ALU dot products instead of the
@@ -230,6 +247,7 @@ NVJ_API int nvj_paged_decode_launch(void* stream,
 #define NVJ_PHASE_VALU_PRODUCTS 4u
 #define NVJ_PHASE_CLEAR_COUNTERS 8u
 #define NVJ_PHASE_LOADS_ONLY 16u
+#define NVJ_PHASE_SHARED_ROWS 32u
 NVJ_API int nvj_paged_decode_launch_phases(void* stream,
                             const void* q, const void* k_cache, const void* v_cache,
                             const int32_t* block_tables, const int32_t* context_lens,
@@ -238,6 +256,51 @@ NVJ_API int nvj_paged_decode_launch_phases(void* stream,
                             int32_t head_dim, int32_t block_size, int32_t max_blocks,
                             int32_t num_blocks, float scale, int32_t chunk, int32_t dtype,
                             uint32_t phases);
+
+/*
+ * The balanced split (chunk == 0) as ONE launch with its counter region and its
+ * partials in separate buffers, so that calls of any shapes can share both: a
+ * counter region stays zero between calls whatever the shapes were.  Stands in
+ * for the same reference call as nvj_paged_decode_launch
+ * (layers/attention.py:389-397); it is the form an XLA custom call uses, with
+ * `partials` an XLA-owned scratch result and counters == NULL.
+ *
+ *   partials  >= nvj_paged_decode_workspace_bytes(.., chunk 0)
+ *                - nvj_paged_decode_counter_bytes(..) bytes, 16-byte aligned,
+ *                contents need not be initialised
+ *   counters  >= nvj_paged_decode_counter_bytes(..) bytes of int32, ZERO before
+ *                the first call (nvj_paged_decode_counters_reset) and left zero
+ *                by every call; or NULL: the library's own region is used, one
+ *                per GPU, 64 KiB (batch * num_kv_heads < 16384, else
+ *                NVJ_ERR_SCRATCH_LIMIT), zero when the library is loaded
+ *
+ *   phases    NVJ_PHASE_SPLITK for the call as described; NVJ_PHASE_CLEAR_COUNTERS
+ *                or-ed in clears the counter region first (a second launch);
+ *                the measurement bits of nvj_paged_decode_launch_phases apply
+ *
+ * Calls that may overlap in time on one GPU must not share a counter region
+ * (with NULL: all such calls, and nvj_paged_decode_static_launch, share the
+ * library's): an overlap loses rows of both calls, and is reported through the
+ * stale flag (word 0 of the region) on a best-effort basis.
+ *
+ * nvj_paged_decode_counters_reset: enqueue a kernel (recordable into a graph)
+ * that sets `counter_bytes` bytes at `counters` to zero, stale flag included;
+ * counters == NULL: the library's own region of the current device.
+ *
+ * nvj_paged_decode_library_counters: device address and size of the library's
+ * own region on the current device, for a caller that wants to read the stale
+ * flag (its first int32) back.  No launch.
+ */
+NVJ_API int nvj_paged_decode_launch_counters(void* stream,
+                            const void* q, const void* k_cache, const void* v_cache,
+                            const int32_t* block_tables, const int32_t* context_lens,
+                            void* out, void* partials, size_t partial_bytes,
+                            void* counters, size_t counter_bytes,
+                            int32_t batch, int32_t num_heads, int32_t num_kv_heads,
+                            int32_t head_dim, int32_t block_size, int32_t max_blocks,
+                            int32_t num_blocks, float scale, int32_t dtype, uint32_t phases);
+NVJ_API int nvj_paged_decode_counters_reset(void* stream, void* counters, size_t counter_bytes);
+NVJ_API int nvj_paged_decode_library_counters(void** counters, size_t* bytes);
 
 /*
  * nvj_paged_decode_launch with chunk == 0 (balanced split) for callers that
@@ -249,20 +312,25 @@ NVJ_API int nvj_paged_decode_launch_phases(void* stream,
  * The split-K partials and counters live in a device array of
  * NVJ_STATIC_SCRATCH_BYTES that is part of the library image: every GPU the
  * library runs on holds its own copy from the first call on that GPU until the
- * process ends.  The counters are zero when the library is loaded and every
- * launch leaves them zero, so the call is a single kernel launch.  The call itself
+ * process ends.  Its first 64 KiB are the library's own counter region (see
+ * nvj_paged_decode_launch_counters): zero when the library is loaded and left
+ * zero by every launch, so the call is a single kernel launch.  The call itself
  * allocates and frees nothing (no hipMalloc / hipFree, no allocating library
  * routine); the first call on a device looks the array's address up once.  The
  * device that `stream` belongs to must be the current device.
  *
  * A problem whose partials (nvj_paged_decode_workspace_bytes(..., chunk 0) minus
  * nvj_paged_decode_counter_bytes) exceed NVJ_STATIC_SCRATCH_BYTES - 64 KiB, or
- * whose counters exceed 64 KiB (batch * num_kv_heads > 16384), is rejected with
+ * whose counter region exceeds 64 KiB (batch * num_kv_heads >= 16384), is rejected with
  * NVJ_ERR_SCRATCH_LIMIT; batch 256 with 32 query heads of 128 dims needs 8.5 MB.  All calls on one GPU
  * share the one array: calls that may overlap in time on the same GPU (two
  * streams, two threads) race on it and must be serialised by the caller; calls
- * on one stream are ordered and safe.  Apart from the counters being zero,
- * nothing in the array has to survive from one call to the next.
+ * on one stream are ordered and safe.  Such a race, or context_lens rewritten
+ * while the kernel runs, can also leave counters of the region non-zero, which
+ * spoils later calls too (rows lost, stale flag set) until
+ * nvj_paged_decode_counters_reset(stream, NULL, 0) has run.  Apart from the
+ * counters being zero, nothing in the array has to survive from one call to
+ * the next.
  */
 #define NVJ_STATIC_SCRATCH_BYTES (16u << 20)
 NVJ_API int nvj_paged_decode_static_launch(void* stream,

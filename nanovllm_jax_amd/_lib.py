@@ -13,7 +13,7 @@ import threading
 _LIB_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), "_native",
                          "libnvj_paged_attn.so")
 
-NVJ_ABI_VERSION = 2
+NVJ_ABI_VERSION = 3
 NVJ_DTYPE_BF16 = 0
 NVJ_DTYPE_F32 = 1
 NVJ_DTYPE_F16 = 2
@@ -40,6 +40,14 @@ SYMBOLS = {
         _c.c_void_p, _c.c_void_p, _c.c_size_t,
         _c.c_int32, _c.c_int32, _c.c_int32, _c.c_int32, _c.c_int32, _c.c_int32,
         _c.c_int32, _c.c_float, _c.c_int32, _c.c_int32, _c.c_uint32]),
+    "nvj_paged_decode_launch_counters": (_c.c_int, [
+        _c.c_void_p, _c.c_void_p, _c.c_void_p, _c.c_void_p, _c.c_void_p, _c.c_void_p,
+        _c.c_void_p, _c.c_void_p, _c.c_size_t, _c.c_void_p, _c.c_size_t,
+        _c.c_int32, _c.c_int32, _c.c_int32, _c.c_int32, _c.c_int32, _c.c_int32,
+        _c.c_int32, _c.c_float, _c.c_int32, _c.c_uint32]),
+    "nvj_paged_decode_counters_reset": (_c.c_int, [_c.c_void_p, _c.c_void_p, _c.c_size_t]),
+    "nvj_paged_decode_library_counters": (_c.c_int, [_c.POINTER(_c.c_void_p),
+                                                     _c.POINTER(_c.c_size_t)]),
     "nvj_paged_decode_static_launch": (_c.c_int, [
         _c.c_void_p, _c.c_void_p, _c.c_void_p, _c.c_void_p, _c.c_void_p, _c.c_void_p,
         _c.c_void_p,
@@ -72,6 +80,7 @@ NVJ_PHASE_COMBINE = 2
 NVJ_PHASE_VALU_PRODUCTS = 4
 NVJ_PHASE_CLEAR_COUNTERS = 8
 NVJ_PHASE_LOADS_ONLY = 16
+NVJ_PHASE_SHARED_ROWS = 32
 
 _lock = threading.Lock()
 _lib = None

@@ -1051,12 +1051,24 @@ __device__ __forceinline__ bool arrive(const DecodeArgs& a, int32_t* counters, i
                                        int r0, int r1, const Cut& cut, int n, int lane) {
   // the partial stores of every lane have reached the device before the count does
   wait_for_stores();
-  int32_t* counter = counters + (int64_t)b * a.num_kv_heads + kvh;
+  // word 0 of the counter region is the stale flag, the counters follow
+  int32_t* counter = counters + 1 + (int64_t)b * a.num_kv_heads + kvh;
   int old = 0;
   if (lane == 0)
     old = __hip_atomic_fetch_add(counter, n, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   old = __builtin_amdgcn_readfirstlane(old);
   const int expected = cut.subrun_of(r1 - 1) - cut.subrun_of(r0) + 1;
+  if (old < 0 || old + n > expected) {
+    // The counter did not start at zero: the region was never cleared, an earlier
+    // launch on it was cut short, or two launches overlap on it.  This row's
+    // output is lost; say so where the host can see it and put the counter
+    // back, so that a launch after this one starts from zero again.
+    if (lane == 0) {
+      __hip_atomic_store(counters, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      __hip_atomic_store(counter, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+    return false;
+  }
   if (old + n != expected) return false;
   // last to arrive: every other partial of the row was acknowledged before its
   // writer's count, which this wave has just seen
@@ -1220,14 +1232,20 @@ __device__ __forceinline__ void merge_row(const DecodeArgs& a, uint4* lds, int b
 template <int D, bool F16, int VG = 0>
 __global__ __launch_bounds__(512) void paged_decode_balanced_kernel(DecodeArgs a, int batch,
                                                                     int num_wgs, int min_steps,
-                                                                    int hpw, int alt_hpw, int shift,
-                                                                    int32_t* counters) {
+                                                                    int hpw, int wr_hpw, int wr_tol,
+                                                                    int shift, int32_t* counters) {
   using H = HeadDim<D>;
   constexpr int NW = 8;
   __shared__ uint4 k_tile[NW][kStep * H::kLdsRowPieces];
   constexpr int kLanesWithDims = D / 32 * 16;   // lanes whose k-group holds real dims
   static_assert(sizeof(uint4) * kStep * H::kLdsRowPieces >= 34 * kLanesWithDims * sizeof(float),
                 "a wave's K tile must hold its partial");
+  // whole-row layout only: the lengths of the batch where any lane can index
+  // them, the order the sequences are dealt to the workgroups in, and per wave
+  // the partial of a piece that has to wait for the rest of its row
+  __shared__ __align__(16) int wr_ctx[kKeptSequences];
+  __shared__ int wr_order[kKeptSequences];
+  __shared__ float wr_parked[NW][34 * kLanesWithDims];
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int lane = threadIdx.x & 63;
   const int g = blockIdx.x;
@@ -1244,8 +1262,6 @@ __global__ __launch_bounds__(512) void paged_decode_balanced_kernel(DecodeArgs a
 #pragma unroll
   for (int k = 0; k < kKeep; ++k) kept_ctx[k] = kept_excl[k] = 0;
   int total = 0, total_kept = 0;
-  const int steps0 = __builtin_amdgcn_readfirstlane(steps_of(0));
-  bool same_steps = true;   // every sequence has steps0 steps
 #pragma unroll
   for (int k = 0; k < kKeep; ++k) {
     if (k * 64 < batch) {
@@ -1254,7 +1270,6 @@ __global__ __launch_bounds__(512) void paged_decode_balanced_kernel(DecodeArgs a
       const int incl = wave_inclusive_scan(n);
       kept_excl[k] = total + incl - n;
       total += __builtin_amdgcn_readlane(incl, 63);
-      same_steps = same_steps && __ballot(k * 64 + lane < batch && n != steps0) == 0ull;
     }
   }
   total_kept = total;
@@ -1262,17 +1277,6 @@ __global__ __launch_bounds__(512) void paged_decode_balanced_kernel(DecodeArgs a
     const int n = steps_of(base + lane);
     total += __builtin_amdgcn_readlane(wave_inclusive_scan(n), 63);
   }
-  // Sequences of one length and exactly one row of `alt_hpw` heads per workgroup
-  // (the host offers alt_hpw only then, and only for a batch whose lengths are
-  // all among the kept ones): with that many heads per workgroup every run is
-  // one whole row, its parts meet in LDS and no partial is ever written, which
-  // beats the better stream of `hpw` heads.  Every wave of the launch takes
-  // the same decision.
-  if (alt_hpw > 0 && same_steps && steps0 >= NW / alt_hpw) hpw = alt_hpw;
-  const int parts = NW / hpw;
-  const int rows_per_seq = a.num_kv_heads / hpw;
-  const int part = wave / hpw;
-  const int h_in_row = wave - part * hpw;
   // No step belongs to an empty sequence: its output row (zeros, 0 / (0 + 1e-9))
   // is written here, sequence b by workgroup b modulo the grid.  The lengths of
   // the first kKeep * 64 sequences are in registers already.
@@ -1292,6 +1296,173 @@ __global__ __launch_bounds__(512) void paged_decode_balanced_kernel(DecodeArgs a
         orow[i] = make_uint4(0u, 0u, 0u, 0u);
     }
   }
+
+  // -------------------------------------------------------------------------
+  // Whole-row layout.  When whole rows can be dealt to the workgroups so that
+  // no workgroup gets more than (1 + wr_tol / 256) times its share of the
+  // steps, no row is shared between workgroups: a row cut between the parts of
+  // one workgroup is put together in LDS, and nothing goes through the
+  // workspace or the counters.  The host offers it (wr_hpw > 0: the KV heads
+  // per workgroup to use) when all lengths are among the kept ones and there
+  // are at least as many rows as workgroups.  Rows are dealt in rounds of
+  // num_wgs, forwards and backwards in turn (row of rank p goes to workgroup
+  // p % num_wgs in an even round, num_wgs - 1 - p % num_wgs in an odd one),
+  // first in the order of the batch - enough for lengths that are equal or
+  // nearly so - and, when that is not balanced and there is more than one
+  // round, by decreasing length, which pairs long rows with short ones.  Every
+  // wave of the launch reads the same lengths and takes the same decision.
+  // -------------------------------------------------------------------------
+  if (wr_hpw > 0 && total > 0) {
+    const int w_hpw = wr_hpw;
+    const int w_rps = a.num_kv_heads / w_hpw;
+    const int rows = batch * w_rps;
+    const int rounds = (rows + num_wgs - 1) / num_wgs;
+    // every wave writes all the lengths itself (the same values from each),
+    // so no wave has to wait for another before it reads them back
+#pragma unroll
+    for (int k = 0; k < kKeep; ++k) wr_ctx[k * 64 + lane] = k * 64 + lane < batch ? kept_ctx[k] : -1;
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    auto steps_at = [&](int seq) { return (wr_ctx[seq] + kStep - 1) / kStep; };
+    // the largest number of steps any workgroup is dealt, `sorted`: through wr_order
+    auto largest_deal = [&](bool sorted) {
+      int worst = 0;
+      for (int w0 = 0; w0 < num_wgs; w0 += 64) {
+        const int w = w0 + lane;
+        int load = 0;
+        for (int t = 0; t < rounds; ++t) {
+          const int p = t * num_wgs + ((t & 1) ? num_wgs - 1 - w : w);
+          if (w < num_wgs && p < rows) {
+            const int rank = p / w_rps;
+            load += steps_at(sorted ? wr_order[rank] : rank);
+          }
+        }
+        worst = max(worst, load);
+      }
+#pragma unroll
+      for (int m = 32; m >= 1; m >>= 1) worst = max(worst, __shfl_xor(worst, m, 64));
+      return __builtin_amdgcn_readfirstlane(worst);
+    };
+    const int64_t budget = (int64_t)w_rps * total * (256 + wr_tol);   // 256 * num_wgs * the limit
+    bool whole_rows = (int64_t)largest_deal(false) * num_wgs * 256 <= budget;
+    bool sorted = false;
+    if (!whole_rows && rounds > 1) {
+      // rank of every sequence by decreasing number of steps, ties in batch
+      // order: two threads per sequence count, over half of the batch each,
+      // the sequences that come before it
+      const int i = threadIdx.x >> 1, half = threadIdx.x & 1;
+      const int ni = i < batch ? steps_at(i) : -1;
+      int before = 0;
+      for (int j4 = half * (kKeptSequences / 8); j4 < (half + 1) * (kKeptSequences / 8); ++j4) {
+        const int4 c4 = reinterpret_cast<const int4*>(wr_ctx)[j4];
+        const int cj[4] = {c4.x, c4.y, c4.z, c4.w};
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+          const int j = 4 * j4 + u;
+          const int nj = cj[u] < 0 ? -1 : (cj[u] + kStep - 1) / kStep;
+          before += (nj > ni || (nj == ni && j < i)) ? 1 : 0;
+        }
+      }
+      before += __builtin_amdgcn_update_dpp(0, before, kDppQuadXor1, 0xF, 0xF, false);
+      if (half == 0) wr_order[before] = i;
+      __syncthreads();
+      sorted = true;
+      whole_rows = (int64_t)largest_deal(true) * num_wgs * 256 <= budget;
+    }
+    if (whole_rows) {
+      const int w_parts = NW / w_hpw;
+      const int part = wave / w_hpw;
+      const int h_in_row = wave - part * w_hpw;
+      // the rows dealt to this workgroup, in the order of the rounds
+      auto dealt_row = [&](int t, int& seq, int& hg, int& ctx) {
+        const int p = t * num_wgs + ((t & 1) ? num_wgs - 1 - g : g);
+        seq = 0; hg = 0; ctx = 0;
+        if (p < rows) {
+          const int rank = p / w_rps;
+          seq = sorted ? wr_order[rank] : rank;
+          hg = p - rank * w_rps;
+          ctx = wr_ctx[seq];
+        }
+        seq = __builtin_amdgcn_readfirstlane(seq);
+        hg = __builtin_amdgcn_readfirstlane(hg);
+        ctx = __builtin_amdgcn_readfirstlane(max(ctx, 0));
+      };
+      int mine = 0;   // steps dealt to this workgroup
+      for (int t = 0; t < rounds; ++t) {
+        int seq, hg, ctx;
+        dealt_row(t, seq, hg, ctx);
+        mine += (ctx + kStep - 1) / kStep;
+      }
+      // the steps are cut into equal runs for the parts; a part's first piece,
+      // when it does not start a row, waits in LDS for the part that does
+      const int xs = (int)((int64_t)part * mine / w_parts);
+      const int xe = (int)((int64_t)(part + 1) * mine / w_parts);
+      f32x4 acc[8];
+#pragma unroll
+      for (int jd = 0; jd < 8; ++jd) acc[jd] = f32x4{0.f, 0.f, 0.f, 0.f};
+      float m_run = kNegBig, l_run = 0.f;
+      bool owes = false;       // acc holds the first piece of a row that goes on in later parts
+      int owed_b = 0, owed_kvh = 0, owed_end = 0;
+      const bool holds_dims = lane < kLanesWithDims;
+      int row_start = 0;
+      for (int t = 0; t < rounds && row_start < xe; ++t) {
+        int seq, hg, ctx;
+        dealt_row(t, seq, hg, ctx);
+        const int nb = (ctx + kStep - 1) / kStep;
+        const int lo = max(xs, row_start), hi = min(xe, row_start + nb);
+        if (lo < hi) {
+          const int st = lo - row_start, en = hi - row_start;
+          const int kvh = hg * w_hpw + h_in_row;
+          const int t0 = __builtin_amdgcn_readfirstlane(st * kStep);
+          const int t1 = __builtin_amdgcn_readfirstlane(min(ctx, en * kStep));
+          if constexpr (VG > 0)
+            compute_segment_valu<VG>(a, k_tile[wave], seq, kvh, t0, t1, lane, acc, m_run, l_run);
+          else if constexpr (VG < 0)
+            compute_segment_loads_only(a, seq, kvh, t0, t1, lane, acc, m_run, l_run);
+          else
+            compute_segment<D, F16>(a, k_tile[wave], seq, kvh, t0, t1, lane, acc, m_run, l_run);
+          if (st > 0) {
+            // the row started in an earlier part: park the piece for it
+            if (holds_dims) {
+              float* slot = wr_parked[wave] + lane;
+#pragma unroll
+              for (int jd = 0; jd < 8; ++jd)
+#pragma unroll
+                for (int e = 0; e < 4; ++e) slot[(4 * jd + e) * kLanesWithDims] = acc[jd][e];
+              slot[32 * kLanesWithDims] = m_run;
+              slot[33 * kLanesWithDims] = l_run;
+            }
+          } else if (en == nb) {
+            write_output<D, F16>(a, seq, kvh, lane, acc, l_run);
+          } else {
+            // the row goes on in the next part(s): this is the run's last segment
+            owes = true; owed_b = seq; owed_kvh = kvh; owed_end = row_start + nb;
+          }
+        }
+        row_start += nb;
+      }
+      __syncthreads();
+      if (owes) {
+        if (holds_dims) {
+          for (int p = part + 1; p < w_parts; ++p) {
+            const int ps = (int)((int64_t)p * mine / w_parts);
+            const int pe = (int)((int64_t)(p + 1) * mine / w_parts);
+            if (ps >= owed_end) break;
+            if (pe > ps)
+              add_partial_from_lds<kLanesWithDims>(wr_parked[p * w_hpw + h_in_row] + lane,
+                                                   a.scale_log2e, acc, m_run, l_run);
+          }
+        }
+        write_output<D, F16>(a, owed_b, owed_kvh, lane, acc, l_run);
+      }
+      return;
+    }
+  }
+  const int parts = NW / hpw;
+  const int rows_per_seq = a.num_kv_heads / hpw;
+  const int part = wave / hpw;
+  const int h_in_row = wave - part * hpw;
   Cut cut;
   cut.axis = rows_per_seq * total;
   cut.shift = shift;
@@ -1592,10 +1763,20 @@ int balanced_heads_per_workgroup(int64_t batch, int num_kv_heads, int64_t max_st
 // fewer than this many 32-position steps.
 constexpr int kMinBalancedSteps = 1;
 
+// Whole rows are dealt to the workgroups when no workgroup gets more than
+// 1 + kWholeRowTolerance / 256 times the mean number of steps.
+constexpr int kWholeRowTolerance = 16;
+
 // Waves per workgroup of the fixed split = KV heads a workgroup covers: the
 // largest of 8, 4, 2, 1 that divides the number of KV heads.
 int waves_per_workgroup(int num_kv_heads) {
   return num_kv_heads % 8 == 0 ? 8 : num_kv_heads % 4 == 0 ? 4 : num_kv_heads % 2 == 0 ? 2 : 1;
+}
+
+// The counter region of the balanced split: word 0 is the stale flag, then one
+// int32 per (sequence, KV head as the kernels walk them); padded to 256 bytes.
+size_t counter_region_bytes(int64_t batch, int64_t kv_heads) {
+  return ((size_t)(batch * kv_heads + 1) * sizeof(int32_t) + 255) / 256 * 256;
 }
 
 // Workspace layout.  Fixed chunks: partials of batch * max_chunks slots, every
@@ -1605,7 +1786,7 @@ int waves_per_workgroup(int num_kv_heads) {
 struct WorkspacePlan {
   int64_t records;  // partial records (one query head each)
   int max_chunks;   // fixed-chunk mode only
-  int num_wgs, hpw, alt_hpw, shift; // balanced mode only
+  int num_wgs, hpw, wr_hpw, shift;  // balanced mode only
   size_t counter_bytes;
   size_t bytes;
 };
@@ -1627,26 +1808,28 @@ bool plan_workspace(int64_t batch, int64_t num_heads, int64_t head_dim, int64_t 
     // (units + 1) * sub-runs must fit 31 bits (Cut): coarser units for a very long axis
     plan->shift = 0;
     while ((((axis >> plan->shift) + 2) * wgs * parts) >> 31) ++plan->shift;
-    // Sequences of equal length need no partials at all when every workgroup's
-    // run is exactly one row.  If 2 heads per workgroup give that (and 4 would
-    // share every row between two workgroups), the kernel takes 2 when it finds
-    // the lengths equal (it reads them anyway).  Both layouts fill the same
-    // workspace: slots * hpw = 8 * workgroups + batch * heads.
-    plan->alt_hpw = 0;
-    const bool alt_fits_cut = plan->shift == 0 && (((2 * axis + 2) * wgs * 2 * parts) >> 31) == 0;
-    if (hpw == 4 && wgs == cus && alt_fits_cut && batch * (num_kv_heads / 2) == wgs &&
-        batch <= kKeptSequences)
-      plan->alt_hpw = 2;
+    // The whole-row layout of the kernel (no partials at all) is offered when the
+    // kernel keeps every length in registers and there is a row for every
+    // workgroup, with as many heads per workgroup as still give that (2 at
+    // least: with 1 the K/V stream of a large launch is a tenth slower).  It
+    // needs no workspace of its own.
+    plan->wr_hpw = 0;
+    if (batch <= kKeptSequences)
+      for (int h = hpw; h >= 2; h /= 2)
+        if (num_kv_heads % h == 0 && batch * (num_kv_heads / h) >= wgs) {
+          plan->wr_hpw = h;
+          break;
+        }
     plan->max_chunks = 0;
     const int64_t slots = wgs * parts + batch * rows_per_seq;
     plan->records = slots * hpw * (num_heads / num_kv_heads);
-    plan->counter_bytes = ((size_t)batch * num_kv_heads * sizeof(int32_t) + 255) / 256 * 256;
+    plan->counter_bytes = counter_region_bytes(batch, num_kv_heads);
     plan->bytes = plan->counter_bytes + (size_t)plan->records * (head_dim + 2) * sizeof(float);
     return true;
   }
   const int64_t mc = (max_blocks * block_size + chunk - 1) / chunk;
   if (batch * mc > INT32_MAX) return false;
-  plan->num_wgs = plan->hpw = plan->alt_hpw = plan->shift = 0;
+  plan->num_wgs = plan->hpw = plan->wr_hpw = plan->shift = 0;
   plan->max_chunks = (int)mc;
   plan->records = batch * mc * num_heads;
   plan->counter_bytes = 0;
@@ -1790,7 +1973,7 @@ int launch_decode(void* stream, const void* q, const void* k_cache, const void* 
     if (chunk == 0) {
       // one launch: the workgroup that completes a sequence merges it
       if (phases & NVJ_PHASE_CLEAR_COUNTERS) {
-        const int n = batch * num_kv_heads;
+        const int n = (int)(plan.counter_bytes / sizeof(int32_t));   // stale flag, counters, padding
         if (nvj::launch(zero_int32_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), s,
                         counters, n) != hipSuccess)
           return NVJ_ERR_LAUNCH;
@@ -1800,7 +1983,9 @@ int launch_decode(void* stream, const void* q, const void* k_cache, const void* 
       hipError_t rc;
 #define NVJ_LAUNCH_BALANCED(DV, F16V, VGV)                                                     \
   rc = nvj::launch(paged_decode_balanced_kernel<DV, F16V, VGV>, grid, dim3(512), s, a, batch, \
-                   plan.num_wgs, kMinBalancedSteps, plan.hpw, plan.alt_hpw, plan.shift, counters)
+                   plan.num_wgs, kMinBalancedSteps, plan.hpw,                      \
+                   (phases & NVJ_PHASE_SHARED_ROWS) ? 0 : plan.wr_hpw, kWholeRowTolerance,    \
+                   plan.shift, counters)
       if (loads_only) NVJ_LAUNCH_BALANCED(128, false, -1);
       else if (valu && group == 4) NVJ_LAUNCH_BALANCED(128, false, 4);
       else if (valu) NVJ_LAUNCH_BALANCED(128, false, 8);
@@ -1867,7 +2052,7 @@ extern "C" size_t nvj_paged_decode_counter_bytes(int32_t batch, int32_t num_head
   if (batch <= 0 || num_heads <= 0 || num_kv_heads <= 0 || num_heads % num_kv_heads != 0) return 0;
   const size_t heads =
       (size_t)num_kv_heads * virtual_heads_per_cache_head(num_heads / num_kv_heads);
-  return ((size_t)batch * heads * sizeof(int32_t) + 255) / 256 * 256;
+  return counter_region_bytes(batch, (int64_t)heads);
 }
 
 extern "C" int nvj_paged_decode_launch(void* stream, const void* q, const void* k_cache,
@@ -1887,15 +2072,19 @@ extern "C" int nvj_paged_decode_launch(void* stream, const void* q, const void* 
 }
 
 // ---------------------------------------------------------------------------
-// Entry point that allocates nothing: the balanced split with its workspace in
-// a file-scope device array instead of caller memory.  The array's name is a
-// host-side stand-in; its device address is looked up once per device
-// (hipGetSymbolAddress) and only that address is ever handed to a kernel.
+// The library's own device array.  Its first kCounterRegion bytes are a counter
+// region of the balanced split that belongs to no caller (the same words
+// whatever the shape of a call: zero when the library is loaded, put back to
+// zero by every launch); the rest is the workspace of the entry point that
+// allocates nothing.  The array's name is a host-side stand-in; its device
+// address is looked up once per device (hipGetSymbolAddress) and only that
+// address is ever handed to a kernel.
 // ---------------------------------------------------------------------------
 static __device__ __align__(256) unsigned char scratch[NVJ_STATIC_SCRATCH_BYTES];
 
 namespace {
 constexpr int kMaxDevices = 64;
+constexpr size_t kCounterRegion = 64u << 10;
 std::atomic<void*> g_scratch_ptr[kMaxDevices];   // per device: address of its copy of `scratch`
 
 // Device address of the current device's copy of `scratch`.
@@ -1914,6 +2103,60 @@ int static_scratch_of_current_device(void** out) {
 }
 }  // namespace
 
+extern "C" int nvj_paged_decode_library_counters(void** counters, size_t* bytes) {
+  if (!counters) return NVJ_ERR_NULL_POINTER;
+  if (bytes) *bytes = kCounterRegion;
+  return static_scratch_of_current_device(counters);
+}
+
+extern "C" int nvj_paged_decode_counters_reset(void* stream, void* counters,
+                                               size_t counter_bytes) {
+  if (!counters) {
+    const int rc = static_scratch_of_current_device(&counters);
+    if (rc != NVJ_OK) return rc;
+    counter_bytes = kCounterRegion;
+  }
+  if (reinterpret_cast<uintptr_t>(counters) & 3u) return NVJ_ERR_ALIGNMENT;
+  if (counter_bytes / sizeof(int32_t) > (size_t)INT32_MAX) return NVJ_ERR_BAD_SHAPE;
+  const int n = (int)(counter_bytes / sizeof(int32_t));
+  if (n == 0) return NVJ_OK;
+  return nvj::launch(zero_int32_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256),
+                     static_cast<hipStream_t>(stream), static_cast<int32_t*>(counters),
+                     n) == hipSuccess
+             ? NVJ_OK
+             : NVJ_ERR_LAUNCH;
+}
+
+extern "C" int nvj_paged_decode_launch_counters(void* stream, const void* q, const void* k_cache,
+                                                const void* v_cache, const int32_t* block_tables,
+                                                const int32_t* context_lens, void* out,
+                                                void* partials, size_t partial_bytes,
+                                                void* counters, size_t counter_bytes,
+                                                int32_t batch, int32_t num_heads,
+                                                int32_t num_kv_heads, int32_t head_dim,
+                                                int32_t block_size, int32_t max_blocks,
+                                                int32_t num_blocks, float scale, int32_t dtype,
+                                                uint32_t phases) {
+  if (batch > 0 && max_blocks > 0) {
+    const size_t need = nvj_paged_decode_counter_bytes(batch, num_heads, num_kv_heads);
+    if (!counters) {
+      // need == 0: invalid arguments, which the launch below reports by name
+      if (need > kCounterRegion) return NVJ_ERR_SCRATCH_LIMIT;
+      if (need > 0) {
+        const int rc = static_scratch_of_current_device(&counters);
+        if (rc != NVJ_OK) return rc;
+      }
+    } else {
+      if (reinterpret_cast<uintptr_t>(counters) & 3u) return NVJ_ERR_ALIGNMENT;
+      if (need > 0 && counter_bytes < need) return NVJ_ERR_WORKSPACE;
+    }
+  }
+  return launch_decode(stream, q, k_cache, v_cache, block_tables, context_lens, out, partials,
+                       partial_bytes, static_cast<int32_t*>(counters), batch, num_heads,
+                       num_kv_heads, head_dim, block_size, max_blocks, num_blocks, scale, 0, dtype,
+                       phases);
+}
+
 extern "C" int nvj_paged_decode_static_launch(void* stream, const void* q, const void* k_cache,
                                               const void* v_cache, const int32_t* block_tables,
                                               const int32_t* context_lens, void* out,
@@ -1921,10 +2164,6 @@ extern "C" int nvj_paged_decode_static_launch(void* stream, const void* q, const
                                               int32_t num_kv_heads, int32_t head_dim,
                                               int32_t block_size, int32_t max_blocks,
                                               int32_t num_blocks, float scale, int32_t dtype) {
-  // The array starts with the counters, in a region of fixed size, so that they
-  // are the same words whatever the shape of a call: zero when the library is
-  // loaded, and put back to zero by every launch.  The partials follow.
-  constexpr size_t kCounterRegion = 64u << 10;
   void* base = nullptr;
   if (batch > 0 && max_blocks > 0) {
     const size_t need = nvj_paged_decode_workspace_bytes(batch, num_heads, head_dim, max_blocks,

@@ -77,12 +77,18 @@ ffi::Error StoreKvcacheImpl(hipStream_t stream, ffi::AnyBuffer key, ffi::AnyBuff
 // split, -1 = whole sequence per workgroup: the workspace result is then unused);
 // results: out [B, Hq, D] in q's dtype and the workspace (u8, sized by
 // nvj_paged_decode_workspace_bytes on the Python side so that XLA owns it).  XLA hands
-// over the workspace uninitialised, so this goes through nvj_paged_decode_launch, which
-// clears the counters of the balanced split with a small kernel of its own first.
+// over the workspace uninitialised.  The balanced split therefore keeps only its
+// partials there and takes its counters from the library's own region (zero between
+// calls by invariant), which makes the call a single launch; the executables of one
+// process must then not run decode calls on two streams of one GPU at the same time
+// (XLA's GPU client runs compute on one stream per device).  The attr
+// library_counters = 0 gives up the invariant instead: the whole workspace goes through
+// nvj_paged_decode_launch, which clears its counters with a small kernel of its own.
 ffi::Error PagedDecodeImpl(hipStream_t stream, ffi::AnyBuffer q, ffi::AnyBuffer k_cache,
                            ffi::AnyBuffer v_cache, ffi::Buffer<ffi::DataType::S32> block_tables,
                            ffi::Buffer<ffi::DataType::S32> context_lens, float scale,
-                           int32_t chunk, ffi::Result<ffi::AnyBuffer> out,
+                           int32_t chunk, int32_t library_counters,
+                           ffi::Result<ffi::AnyBuffer> out,
                            ffi::ResultBuffer<ffi::DataType::U8> workspace) {
   const auto qd = q.dimensions();
   const auto cd = k_cache.dimensions();
@@ -93,6 +99,13 @@ ffi::Error PagedDecodeImpl(hipStream_t stream, ffi::AnyBuffer q, ffi::AnyBuffer 
   if (k_cache.element_type() != q.element_type() || v_cache.element_type() != q.element_type() ||
       out->element_type() != q.element_type())
     return bad("q, k_cache, v_cache and out must have one dtype");
+  if (chunk == 0 && library_counters != 0)
+    return to_error(nvj_paged_decode_launch_counters(
+        stream, q.untyped_data(), k_cache.untyped_data(), v_cache.untyped_data(),
+        block_tables.typed_data(), context_lens.typed_data(), out->untyped_data(),
+        workspace->typed_data(), workspace->size_bytes(), nullptr, 0, (int32_t)qd[0],
+        (int32_t)qd[1], (int32_t)cd[2], (int32_t)qd[2], (int32_t)cd[1], (int32_t)td[1],
+        (int32_t)cd[0], scale, code, NVJ_PHASE_SPLITK));
   return to_error(nvj_paged_decode_launch(
       stream, q.untyped_data(), k_cache.untyped_data(), v_cache.untyped_data(),
       block_tables.typed_data(), context_lens.typed_data(), out->untyped_data(),
@@ -127,6 +140,7 @@ XLA_FFI_DEFINE_HANDLER_SYMBOL(
         .Arg<ffi::Buffer<ffi::DataType::S32>>()
         .Attr<float>("scale")
         .Attr<int32_t>("chunk")
+        .Attr<int32_t>("library_counters")
         .Ret<ffi::AnyBuffer>()
         .Ret<ffi::Buffer<ffi::DataType::U8>>(),
     {ffi::Traits::kCmdBufferCompatible});

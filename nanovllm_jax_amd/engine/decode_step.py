@@ -208,6 +208,8 @@ class DecodeStepRunner:
             a.set_kv_cache(self.kv_cache[0, layer], self.kv_cache[1, layer])
             self.attn.append(a)
         self._graph = None
+        self._eager_ws = None
+        self._eager_ws_shapes = set()
 
     # -- small torch pieces -------------------------------------------------
     def _rms(self, x, weight, residual=None):
@@ -275,7 +277,8 @@ class DecodeStepRunner:
                 else:
                     o = paged_attention(q, attn.k_cache, attn.v_cache, context.block_tables,
                                         context.context_lens, attn.scale, attn.block_size,
-                                        chunk=context.decode_split, workspace=attn.workspace)
+                                        chunk=context.decode_split,
+                                        workspace=attn.workspace or self._eager_workspace(context))
                 h = F.linear(o.reshape(-1, qs), lw["o"])
                 h, residual = self._rms(h, lw["ln2"], residual)
                 h = F.linear(self._silu_mul(F.linear(h, lw["gate_up"])), lw["down"])
@@ -324,67 +327,78 @@ class DecodeStepRunner:
         """Eager decode step: logits -> greedy token ids [batch] int64."""
         return self.forward(input_ids, positions, context).argmax(dim=-1)
 
-    def _share_workspace(self, batch, max_blocks, decode_split):
-        """One split workspace for all layers (they run one after the other on
-        one stream), large enough for the balanced split and for the split the
-        context asks for; its counters are zero from the start."""
+    def _eager_workspace(self, context):
+        """The split workspace of the eager steps (one stream), grown on demand."""
+        batch, max_blocks = context.block_tables.shape
+        key = (batch, max_blocks, int(context.decode_split))
+        if key not in self._eager_ws_shapes:
+            ws = self._new_workspace(*key)
+            if self._eager_ws is None or ws.buffer.numel() > self._eager_ws.buffer.numel():
+                self._eager_ws = ws
+            self._eager_ws_shapes.add(key)
+        return self._eager_ws
+
+    def _new_workspace(self, batch, max_blocks, decode_split):
+        """A split workspace for all layers of one step (they run one after the
+        other on one stream), large enough for the balanced split and for the
+        split the context asks for; its counters are zero from the start."""
         c = self.cfg
         with torch.cuda.device(self.device):
             need = max(paged_decode_workspace_bytes(batch, c.num_heads, c.head_dim, max_blocks,
                                                     c.block_size, c.num_kv_heads, chunk)
                        for chunk in {0, int(decode_split)})
-        ws = DecodeWorkspace(need, self.device)
-        for a in self.attn:
-            a.workspace = ws
+        return DecodeWorkspace(need, self.device)
 
-    def capture(self, input_ids, positions, context):
-        """Capture the whole step in one HIP graph over static input buffers;
-        returns ``replay() -> token ids`` (the inputs may be updated in place
-        between replays)."""
-        c = self.cfg
+    def _capture(self, input_ids, positions, context, body, warmups):
+        """Record ``body()`` into a HIP graph.  The graph gets a split workspace of
+        its own, which stays alive with the returned closure and is never handed
+        to an eager call: a replay can then rely on counters that nothing but
+        its own launches has touched, whatever eager steps (of any batch size)
+        or further captures run in between."""
         batch, max_blocks = context.block_tables.shape
-        self._share_workspace(batch, max_blocks, context.decode_split)
-        s = torch.cuda.Stream(self.device)
-        s.wait_stream(torch.cuda.current_stream(self.device))
-        with torch.cuda.stream(s):
-            for _ in range(2):
-                self.step(input_ids, positions, context)
-        torch.cuda.current_stream(self.device).wait_stream(s)
-        torch.cuda.synchronize()
-        graph = torch.cuda.CUDAGraph()
-        with torch.cuda.graph(graph):
-            out = self.step(input_ids, positions, context)
+        graph_ws = self._new_workspace(batch, max_blocks, context.decode_split)
+        eager_ws = [a.workspace for a in self.attn]
+        for a in self.attn:
+            a.workspace = graph_ws
+        try:
+            # warm every library handle on a side stream; a warm-up step writes the
+            # K/V rows of the current step, which the captured step rewrites with
+            # the same values, and does not touch the metadata
+            s = torch.cuda.Stream(self.device)
+            s.wait_stream(torch.cuda.current_stream(self.device))
+            with torch.cuda.stream(s):
+                for _ in range(warmups):
+                    self.step(input_ids, positions, context)
+            torch.cuda.current_stream(self.device).wait_stream(s)
+            torch.cuda.synchronize()
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph):
+                out = body()
+        finally:
+            for a, ws in zip(self.attn, eager_ws):
+                a.workspace = ws
         self._graph = graph
 
         def replay():
             graph.replay()
             return out
+        replay.workspace = graph_ws      # keeps it alive; also lets a caller check() it
         return replay
+
+    def capture(self, input_ids, positions, context):
+        """Capture the whole step in one HIP graph over static input buffers;
+        returns ``replay() -> token ids`` (the inputs may be updated in place
+        between replays)."""
+        return self._capture(input_ids, positions, context,
+                             lambda: self.step(input_ids, positions, context), 2)
 
     def capture_generation(self, input_ids, positions, context):
         """Capture step + metadata advance in one HIP graph: every replay decodes
         one token per sequence and leaves ``input_ids / positions / context``
         ready for the next replay, with nothing but block-table maintenance left
         to the host.  Returns ``replay() -> token ids of that step``."""
-        c = self.cfg
-        batch, max_blocks = context.block_tables.shape
-        self._share_workspace(batch, max_blocks, context.decode_split)
-        # warm every library handle on a side stream; the warm-up step writes
-        # the K/V rows of the current step, which the captured step rewrites
-        # with the same values, and does not touch the metadata
-        s = torch.cuda.Stream(self.device)
-        s.wait_stream(torch.cuda.current_stream(self.device))
-        with torch.cuda.stream(s):
-            self.step(input_ids, positions, context)
-        torch.cuda.current_stream(self.device).wait_stream(s)
-        torch.cuda.synchronize()
-        graph = torch.cuda.CUDAGraph()
-        with torch.cuda.graph(graph):
+        def body():
             out = self.step(input_ids, positions, context)
-            advance_decode(out, input_ids, positions, context, c.block_size)
-        self._graph = graph
-
-        def replay():
-            graph.replay()
+            advance_decode(out, input_ids, positions, context, self.cfg.block_size)
             return out
-        return replay
+        return self._capture(input_ids, positions, context, body, 1)

@@ -58,20 +58,23 @@ def paged_decode_workspace_bytes(batch: int, num_heads: int, head_dim: int,
 class DecodeWorkspace:
     """Split workspace kept across the decode calls of ONE stream.
 
-    The balanced split (``chunk=0``) merges the partials of a sequence inside
-    its one launch, by way of counters at the head of the workspace that must be
-    zero when a launch starts and are zero again when it ends.  This buffer is
-    zeroed when it is created, so a call that is handed a ``DecodeWorkspace`` is
-    a single kernel launch; a plain tensor (contents unknown) costs a small
-    clearing launch in front of every call.  Calls that may overlap in time
-    (different streams) need a workspace each."""
+    The balanced split (``chunk=0``) merges the partials of a shared row inside
+    its one launch, by way of counters that must be zero when a launch starts
+    and are zero again when it ends.  Here the counters live in a buffer of
+    their own, zeroed when it is created and apart from the partials, so calls
+    of any shapes can share one ``DecodeWorkspace`` and each is a single kernel
+    launch (``nvj_paged_decode_launch_counters``); a plain tensor (contents
+    unknown) costs a small clearing launch in front of every call.  Calls that
+    may overlap in time (different streams, a captured graph and eager calls)
+    need a workspace each."""
 
-    def __init__(self, nbytes: int, device):
-        self.buffer = torch.zeros(max(int(nbytes), 16), dtype=torch.uint8, device=device)
-        # bytes from the start known to be zero: everything at first, afterwards
-        # the counters of the last call (a launch puts exactly those back to zero;
-        # behind them lie its partials)
-        self.zero_prefix = self.buffer.numel()
+    COUNTER_BYTES = 64 << 10
+
+    def __init__(self, nbytes: int, device, counter_bytes: int = COUNTER_BYTES):
+        self.buffer = torch.empty(max(int(nbytes), 16), dtype=torch.uint8, device=device)
+        self.counters = torch.zeros(max(int(counter_bytes), 256) // 4, dtype=torch.int32,
+                                    device=device)
+        self._clear_next = False
 
     @classmethod
     def for_shape(cls, batch: int, num_heads: int, head_dim: int, max_blocks: int,
@@ -79,7 +82,26 @@ class DecodeWorkspace:
         with torch.cuda.device(device):   # the size follows the device's CU count
             need = paged_decode_workspace_bytes(batch, num_heads, head_dim, max_blocks,
                                                 block_size, num_kv_heads, chunk)
-        return cls(need, device)
+            counters = int(_lib.load().nvj_paged_decode_counter_bytes(batch, num_heads,
+                                                                      num_kv_heads))
+        return cls(need, device, max(counters, cls.COUNTER_BYTES))
+
+    def _counters_for(self, nbytes: int) -> torch.Tensor:
+        if nbytes > self.counters.numel() * 4:
+            self.counters = torch.zeros(-(-nbytes // 256) * 64, dtype=torch.int32,
+                                        device=self.counters.device)
+        return self.counters
+
+    def check(self) -> bool:
+        """Synchronises, then reads the stale flag of the counters: False when a
+        launch since the last check found a counter that did not start at zero
+        (an earlier launch cut short, two launches overlapping on this
+        workspace) and so lost rows of its output.  The counters are then
+        cleared in front of the next call."""
+        ok = int(self.counters[0].item()) == 0
+        if not ok:
+            self._clear_next = True
+        return ok
 
 
 def _compute_units(device=None) -> int:
@@ -212,7 +234,7 @@ def paged_attention(q, k_cache, v_cache, block_tables, context_lens, scale, bloc
              and block_tables.is_contiguous() and context_lens.is_contiguous(),
              "q, k_cache, v_cache, block_tables and context_lens must be contiguous")
     (dev_index, batch, num_heads, num_kv_heads, head_dim, bs, max_blocks, num_blocks, need,
-     counters, dtype_code) = plan
+     counter_bytes, dtype_code) = plan
     dev = q.device
 
     if out is None:
@@ -222,13 +244,14 @@ def paged_attention(q, k_cache, v_cache, block_tables, context_lens, scale, bloc
                  and out.device == dev and out.is_contiguous(),
                  "out must be a contiguous tensor matching q")
     phases = int(phases)
+    counters = None
     if isinstance(workspace, DecodeWorkspace):
-        # its counters are zero between calls, unless a call of a smaller shape
-        # has since written partials where this call's counters lie
-        if counters > workspace.zero_prefix:
-            phases |= _lib.NVJ_PHASE_CLEAR_COUNTERS
-        if chunk >= 0 and need:
-            workspace.zero_prefix = counters
+        if chunk == 0 and need:
+            counters = workspace._counters_for(counter_bytes)
+            if workspace._clear_next:
+                phases |= _lib.NVJ_PHASE_CLEAR_COUNTERS
+                workspace._clear_next = False
+            need -= counter_bytes           # the buffer holds the partials only
         workspace = workspace.buffer
     else:
         phases |= _lib.NVJ_PHASE_CLEAR_COUNTERS
@@ -241,6 +264,14 @@ def paged_attention(q, k_cache, v_cache, block_tables, context_lens, scale, bloc
     _require(ws_bytes >= need, f"workspace too small: need {need} bytes")
 
     def launch():
+        if counters is not None:
+            _require(counters.device == dev, "the workspace's counters are on another device")
+            return lib.nvj_paged_decode_launch_counters(
+                _raw_stream(dev_index), q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(),
+                block_tables.data_ptr(), context_lens.data_ptr(), out.data_ptr(),
+                workspace.data_ptr(), ws_bytes, counters.data_ptr(), counters.numel() * 4,
+                batch, num_heads, num_kv_heads, head_dim, bs, max_blocks, num_blocks,
+                float(scale), dtype_code, phases)
         return lib.nvj_paged_decode_launch_phases(
             _raw_stream(dev_index), q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(),
             block_tables.data_ptr(), context_lens.data_ptr(), out.data_ptr(),
@@ -253,5 +284,6 @@ def paged_attention(q, k_cache, v_cache, block_tables, context_lens, scale, bloc
         with torch.cuda.device(dev_index):
             code = launch()
     if code != 0:
-        _lib.check(code, "nvj_paged_decode_launch_phases")
+        _lib.check(code, "nvj_paged_decode_launch_counters" if counters is not None
+                   else "nvj_paged_decode_launch_phases")
     return out

@@ -120,6 +120,27 @@ def make_workload(name: str, seed: int | None = None) -> DecodeWorkload:
         ctx = rng.integers(200, 2048, size=B).astype(np.int32)
         bt = np.arange(NB, dtype=np.int32).reshape(B, MB)
         gain = 1.0
+    elif name in ("C2_JITTER", "C2_SPREAD", "RAGGED_SHORT"):
+        # batches as a serving loop really sees them (the reference's filler hands over
+        # whatever lengths the running sequences have, engine/model_runner.py:357-361):
+        # C2 with lengths a few percent apart, C2 with lengths from half to one and a
+        # half times 4096, and 256 short sequences of 200 to 2048 positions
+        seed = {"C2_JITTER": 1012, "C2_SPREAD": 1022, "RAGGED_SHORT": 1032}[name] \
+            if seed is None else seed
+        rng = np.random.Generator(np.random.PCG64(seed))
+        Hq, Hkv, D, bs = 32, 8, 128, 256
+        if name == "C2_JITTER":
+            B, ctx = 64, rng.integers(3840, 4097, size=64)
+        elif name == "C2_SPREAD":
+            B, ctx = 64, rng.integers(2048, 6145, size=64)
+        else:
+            B, ctx = 256, rng.integers(200, 2049, size=256)
+        ctx = ctx.astype(np.int32)
+        nblk = -(-ctx // bs)
+        NB = int(np.ceil(1.1 * nblk.sum()))
+        MB = int(nblk.max())
+        bt = _tables_from_counts(rng, nblk, NB, MB)
+        gain = 1.0
     else:
         raise KeyError(name)
     return DecodeWorkload(name=name, batch=B, num_heads=Hq, num_kv_heads=Hkv,
@@ -128,7 +149,7 @@ def make_workload(name: str, seed: int | None = None) -> DecodeWorkload:
                           slot_mapping=_slots(bt, ctx, bs), q_gain=gain, seed=seed)
 
 
-WORKLOADS = ("C1", "C2", "C3", "C4", "C5", "R1")
+WORKLOADS = ("C1", "C2", "C3", "C4", "C5", "R1", "C2_JITTER", "C2_SPREAD", "RAGGED_SHORT")
 
 
 def draw_bf16_bits(rng: np.random.Generator, shape, gain: float = 1.0) -> np.ndarray:

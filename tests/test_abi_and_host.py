@@ -73,12 +73,27 @@ def test_argument_validation_without_a_gpu():
     assert P(None, x, x, x, x, x, x, x, 1 << 30, 2, 8, 2, 64, 256, 4, 16, 0.1, 0, 0, lo) == -3
     assert P(None, x, x, x, x, x, x, x, 1 << 30, 2, 32, 8, 128, 256, 4, 16, 0.1, 0, 0,
              lo | _lib.NVJ_PHASE_VALU_PRODUCTS) == -3
-    # counters of the balanced split: one int32 per (sequence, KV head as the kernels walk
-    # them: a group above 16 query heads counts as several), padded to 256 bytes
+    # counter region of the balanced split: the stale flag, then one int32 per (sequence,
+    # KV head as the kernels walk them: a group above 16 query heads counts as several),
+    # padded to 256 bytes
     C = lib.nvj_paged_decode_counter_bytes
-    assert C(64, 32, 8) == 2048 and C(1, 8, 8) == 256 and C(3, 32, 1) == 256
-    assert C(100, 64, 2) == 1792          # 100 x (2 cache heads x 2 virtual heads of 16) x 4 B, padded
+    assert C(64, 32, 8) == 2304 and C(1, 8, 8) == 256 and C(3, 32, 1) == 256
+    assert C(100, 64, 2) == 1792          # (1 + 100 x 2 cache heads x 2 virtual heads of 16) x 4 B, padded
     assert C(0, 32, 8) == 0 and C(4, 30, 8) == 0
+    # the balanced split with its counters apart from its partials
+    LC = lib.nvj_paged_decode_launch_counters
+    one = _lib.NVJ_PHASE_SPLITK
+    assert LC(None, x, x, x, x, x, x, x, 1 << 30, x, 1 << 16, 2, 32, 8, 96, 256, 4, 16, 0.1, 0, one) == -3
+    assert LC(None, x, x, x, x, x, x, x, 1 << 30, x, 16, 2, 32, 8, 128, 256, 4, 16, 0.1, 0, one) == -4
+    assert LC(None, x, x, x, x, x, x, x, 16, x, 1 << 16, 2, 32, 8, 128, 256, 4, 16, 0.1, 0, one) == -4
+    assert LC(None, x, x, x, x, x, x, x, 1 << 30, x + 2, 1 << 16, 2, 32, 8, 128, 256, 4, 16, 0.1, 0,
+              one) == -8
+    assert LC(None, x, x, x, x, x, x, x, 1 << 30, x, 1 << 16, 0, 32, 8, 128, 256, 4, 16, 0.1, 0, one) == 0
+    # the library's own counter region holds 16383 counters
+    assert LC(None, x, x, x, x, x, x, x, 1 << 30, None, 0, 2048, 8, 8, 128, 256, 4, 16, 0.1, 0,
+              one) == -7
+    R = lib.nvj_paged_decode_counters_reset
+    assert R(None, x + 1, 64) == -8 and R(None, x, 0) == 0
     PP = lib.nvj_paged_prefill_attention_launch
     assert PP(None, x, x, x, x, x, x, x, 10, 2, 32, 8, 128, 48, 4, 16, 0.1, 0) == -3   # page % 32
     assert PP(None, x, x, x, x, x, x, x, 10, 2, 32, 8, 64, 64, 4, 16, 0.1, 0) == -3    # head_dim
@@ -108,7 +123,7 @@ def test_workspace_and_chunk_queries():
     # a workgroup is 4 KV heads x 2 parts, at batch 2 it is 2 KV heads x 4 parts, and 1 KV
     # head x 8 parts for a single long sequence
     assert paged_decode_workspace_bytes(64, 32, 128, 16, 256, 8, 0) == \
-        2048 + (256 * 2 + 64 * 2) * 4 * 4 * (128 + 2) * 4
+        2304 + (256 * 2 + 64 * 2) * 4 * 4 * (128 + 2) * 4
     assert paged_decode_workspace_bytes(2, 8, 128, 1, 32, 8, 0) == 256 + (2 * 4 + 2 * 4) * 2 * 130 * 4
     assert paged_decode_workspace_bytes(1, 8, 128, 32, 256, 8, 0) == 256 + (256 * 8 + 8) * 130 * 4
 

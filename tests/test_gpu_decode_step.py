@@ -120,6 +120,46 @@ def test_graph_replays_match_eager_step():
         assert torch.equal(again, eager_tokens)
 
 
+def test_captured_graph_keeps_a_workspace_of_its_own():
+    """A captured step must not share its split workspace with eager steps or with
+    other captures: an eager step of another batch size, and a second capture, between
+    two replays leave the first graph's replays equal to the eager step of its batch.
+    Ragged lengths, so rows are shared between workgroups and the counters are in use."""
+    print("case captured graph owns its workspace", flush=True)
+    from nanovllm_jax_amd.engine.decode_step import DecodeModelConfig, DecodeStepRunner
+    cfg = DecodeModelConfig(num_layers=2, hidden_size=256, num_heads=4, num_kv_heads=2,
+                            head_dim=128, intermediate_size=512, vocab_size=1024,
+                            max_position=4096, block_size=256, num_kvcache_blocks=160)
+    runner = DecodeStepRunner(cfg, "cuda:0", seed=5)
+    rng = np.random.Generator(np.random.PCG64(21))
+    lens = rng.integers(40, 1500, size=24).tolist()
+    lens[3], lens[17] = 3000, 2600
+    pages = rng.permutation(cfg.num_kvcache_blocks).tolist()
+    tables, off = [], 0
+    for n in lens:
+        k = -(-n // cfg.block_size)
+        tables.append(pages[off:off + k]); off += k
+    last = rng.integers(0, cfg.vocab_size, len(lens)).tolist()
+    big = runner.make_inputs(last, lens, tables)
+    small = runner.make_inputs(last[:10], lens[:10], tables[:10])
+    want_big = runner.step(*big).clone()
+    want_small = runner.step(*small).clone()
+    torch.cuda.synchronize()
+    replay_big = runner.capture(*big)
+    assert torch.equal(replay_big(), want_big)
+    assert torch.equal(runner.step(*small), want_small)      # eager, another batch size
+    assert torch.equal(replay_big(), want_big)
+    replay_small = runner.capture(*small)                    # a second capture
+    assert torch.equal(replay_small(), want_small)
+    assert torch.equal(replay_big(), want_big)
+    assert torch.equal(runner.step(*big), want_big)
+    assert torch.equal(replay_small(), want_small)
+    torch.cuda.synchronize()
+    assert replay_big.workspace is not replay_small.workspace
+    assert replay_big.workspace.check() and replay_small.workspace.check()
+    assert runner._eager_ws.check()
+
+
 def test_advance_decode_matches_oracle_over_many_steps():
     """Device-resident metadata advance, bit-exact against the oracle, with the
     host only maintaining the block tables."""

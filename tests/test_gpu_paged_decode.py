@@ -254,42 +254,316 @@ def test_balanced_split_every_workgroup_shape(B, Hq, Hkv, D, lo, hi):
     assert not got[ctx == 0].any()
 
 
-@pytest.mark.parametrize("odd_one", [None, 3, 100])
-def test_balanced_split_layout_chosen_on_the_device(odd_one):
-    """128 sequences x 4 KV heads of 8 steps each: the host plans 4 KV heads per
-    workgroup (128 rows, each shared by two of the 256 workgroups); the kernel finds
-    the step counts equal and takes 2 KV heads instead (256 rows, one whole row per
-    workgroup, merged in LDS): nothing is written to the workspace.  With one
-    shorter sequence it must stay with the host's plan, and partials appear.  Both
-    against the oracle."""
-    print(f"case device-chosen layout odd_one={odd_one}", flush=True)
-    B, Hq, Hkv, D, bs = 128, 8, 4, 128, 64
-    rng = np.random.Generator(np.random.PCG64(77))
-    ctx = rng.integers(250, 257, size=B)        # 8 steps of 32 each
-    if odd_one is not None:
-        ctx[odd_one] = 100                      # 4 steps
-    NB = int((-(-ctx // bs)).sum()) + 2
-    q, kc, vc, bt, ctx = make_problem(4242, B, Hq, Hkv, D, bs, NB, ctx)
-    scale = 1.0 / np.sqrt(D)
+def _steps(ctx, cap):
+    return -(-np.clip(np.asarray(ctx, np.int64), 0, cap) // 32)
+
+
+def deals_whole_rows(ctx, num_kv_heads, table_positions, cus=256, tolerance=16):
+    """The balanced kernel's own layout rule, restated: are whole (sequence, head
+    group) rows dealt to the workgroups (nothing shared, workspace untouched)?
+    Returns (whole_rows, sorted): `sorted` when it took the order by decreasing
+    length to get there."""
+    B = len(ctx)
+    max_steps = -(-table_positions // 32)
+    hpw = 2
+    if B * num_kv_heads <= 16 and max_steps >= 192:
+        hpw = 1
+    elif B >= 32 or (B >= 16 and max_steps >= 128):
+        hpw = 4
+    while hpw > 1 and num_kv_heads % hpw:
+        hpw //= 2
+    axis = (num_kv_heads // hpw) * B * max_steps
+    wgs = min(cus, max(1, -(-axis // (8 // hpw))))
+    wr = 0
+    h = hpw
+    while B <= 256 and h >= 2:
+        if num_kv_heads % h == 0 and B * (num_kv_heads // h) >= wgs:
+            wr = h
+            break
+        h //= 2
+    steps = _steps(ctx, table_positions)
+    if wr == 0 or steps.sum() == 0:
+        return False, False
+    rps = num_kv_heads // wr
+    rows = B * rps
+    rounds = -(-rows // wgs)
+
+    def largest(order):
+        load = np.zeros(wgs, np.int64)
+        for p in range(rows):
+            t, w = divmod(p, wgs)
+            load[wgs - 1 - w if t % 2 else w] += steps[order[p // rps]]
+        return int(load.max())
+
+    budget = rps * int(steps.sum()) * (256 + tolerance)
+    if largest(np.arange(B)) * wgs * 256 <= budget:
+        return True, False
+    if rounds > 1 and largest(np.argsort(-steps, kind="stable")) * wgs * 256 <= budget:
+        return True, True
+    return False, False
+
+
+def _run_over_marked_workspace(q, kc, vc, bt, ctx, scale, bs, extra_phases=0):
+    """A chunk = 0 call over a workspace full of ones: returns the output and whether
+    the partials are still all ones afterwards (then no row was shared)."""
     import torch
     from nanovllm_jax_amd import _lib, paged_attention
     from nanovllm_jax_amd.layers.paged_attention import paged_decode_workspace_bytes
     dev = "cuda:0"
-    # a workspace full of ones: whatever is still all ones afterwards was not written
+    B, Hq, D = q.shape
+    Hkv = kc.shape[2]
     ws = torch.full((paged_decode_workspace_bytes(B, Hq, D, bt.shape[1], bs, Hkv, 0),), 0xFF,
                     dtype=torch.uint8, device=dev)
     out = paged_attention(bits_to_torch(q, dev), bits_to_torch(kc, dev), bits_to_torch(vc, dev),
                           torch.from_numpy(bt).to(dev), torch.from_numpy(ctx).to(dev), scale, bs,
-                          chunk=0, workspace=ws)
+                          chunk=0, workspace=ws,
+                          phases=_lib.NVJ_PHASE_SPLITK | _lib.NVJ_PHASE_COMBINE | extra_phases)
     torch.cuda.synchronize()
-    want = oracle(q, kc, vc, bt, ctx, scale, bs)
-    assert_close_bf16(torch_to_bits(out), want, what=f"device-chosen layout odd_one={odd_one}")
     counters = int(_lib.load().nvj_paged_decode_counter_bytes(B, Hq, Hkv))
-    assert not ws[:counters].any(), "counters are zero after the call"
-    partials_untouched = bool((ws[counters:] == 0xFF).all())
-    assert partials_untouched == (odd_one is None), \
-        "equal step counts: no partial is written; one odd sequence: some are"
+    assert not ws[:counters].any(), "the counter region is zero after the call"
+    return torch_to_bits(out), bool((ws[counters:] == 0xFF).all())
 
+
+@pytest.mark.parametrize("name", ["equal", "within_tolerance", "one_short", "one_long",
+                                  "pairs_by_length", "pairs_four_rounds", "log_uniform",
+                                  "equal_forced_shared"])
+def test_balanced_split_deals_whole_rows_when_that_is_balanced(name):
+    """The kernel looks at the lengths and, when whole rows can be dealt to the
+    workgroups within 1/16 of an equal share, shares no row (the workspace stays
+    untouched): equal lengths; lengths a few percent apart; one short sequence among
+    equal ones; lengths that only balance when long rows are paired with short ones
+    (the order by decreasing length, two and four rounds of rows).  It must not do so
+    when one long sequence or a log-uniform spread would leave workgroups idle, and
+    not when the caller forbids it.  Every case against the oracle, and the layout
+    against the rule restated in deals_whole_rows."""
+    print(f"case whole rows {name}", flush=True)
+    from nanovllm_jax_amd import _lib
+    rng = np.random.Generator(np.random.PCG64(len(name) * 131 + 5))
+    bs, extra = 64, 0
+    if name in ("equal", "equal_forced_shared", "within_tolerance", "one_short", "one_long"):
+        B, Hq, Hkv, D = 128, 8, 4, 128                 # 128 rows of 4 heads, 256 rows of 2
+        ctx = {"equal": lambda: rng.integers(930, 961, size=B),            # 30 steps each
+               "equal_forced_shared": lambda: rng.integers(930, 961, size=B),
+               "within_tolerance": lambda: rng.integers(870, 961, size=B),  # 28..30 steps
+               "one_short": lambda: np.where(np.arange(B) == 77, 100, 960),
+               "one_long": lambda: np.where(np.arange(B) == 77, 2900, 960)}[name]()
+        if name == "equal_forced_shared":
+            extra = _lib.NVJ_PHASE_SHARED_ROWS
+    elif name == "pairs_by_length":
+        B, Hq, Hkv, D = 256, 8, 8, 64                  # 512 rows of 4 heads: two rounds
+        ctx = rng.integers(64, 1400, size=B)
+    elif name == "pairs_four_rounds":
+        B, Hq, Hkv, D = 256, 16, 16, 64                # 1024 rows of 4 heads: four rounds
+        ctx = rng.integers(64, 1000, size=B)
+    else:
+        B, Hq, Hkv, D = 256, 8, 8, 64
+        ctx = np.rint(np.exp(rng.uniform(np.log(16.0), np.log(4096.0), size=B))).astype(np.int64)
+    NB = int((-(-ctx // bs)).sum()) + 2
+    q, kc, vc, bt, ctx = make_problem(4242 + B, B, Hq, Hkv, D, bs, NB, ctx)
+    scale = 1.0 / np.sqrt(D)
+    got, untouched = _run_over_marked_workspace(q, kc, vc, bt, ctx, scale, bs, extra)
+    assert_close_bf16(got, oracle(q, kc, vc, bt, ctx, scale, bs), what=f"whole rows {name}")
+    whole, by_length = deals_whole_rows(ctx, Hkv, bt.shape[1] * bs)
+    expect = {"equal": (True, False), "within_tolerance": (True, False),
+              "one_short": (True, False), "one_long": (False, False),
+              "pairs_by_length": (True, True), "pairs_four_rounds": (True, True),
+              "log_uniform": (False, False), "equal_forced_shared": (True, False)}[name]
+    assert (whole, by_length) == expect, "the case does not exercise what its name says"
+    assert untouched == (whole and not extra), \
+        f"{name}: partials {'untouched' if untouched else 'written'}"
+
+
+def test_balanced_split_whole_rows_equal_the_shared_rows_split():
+    """The two layouts of chunk = 0 on one batch each: same result to fp32 round-off of
+    the merge order (far inside the bar), for bf16 and float16, head_dim 128 and 64, a
+    group of 16, and a batch with empty sequences in it."""
+    import torch
+    from nanovllm_jax_amd import _lib, paged_attention
+    from oracle.paged_attention_oracle import bf16_bits_to_f32
+    dev = "cuda:0"
+    for seed, B, Hq, Hkv, D, lo, hi, dt in [(1, 64, 32, 8, 128, 1000, 1024, torch.bfloat16),
+                                            (2, 128, 16, 8, 64, 400, 420, torch.float16),
+                                            (3, 256, 32, 2, 128, 200, 224, torch.bfloat16),
+                                            (4, 128, 16, 16, 64, 0, 1200, torch.bfloat16)]:
+        print(f"case both layouts seed={seed} B={B} Hq={Hq} Hkv={Hkv} D={D} {dt}", flush=True)
+        rng = np.random.Generator(np.random.PCG64(seed))
+        bs = 32
+        ctx = rng.integers(lo, hi + 1, size=B)
+        if lo == 0:
+            # short and empty sequences, each with a partner that makes up the difference
+            half = rng.integers(0, hi // 32 + 1, size=B // 2) * 32
+            half[rng.integers(0, B // 2, size=20)] = 0
+            ctx = rng.permutation(np.concatenate([half, 2 * hi - half]))
+        q, kc, vc, bt, ctx = make_problem(50 + seed, B, Hq, Hkv, D, bs,
+                                          int((-(-ctx // bs)).sum()) + 1, ctx)
+        assert deals_whole_rows(ctx, Hkv * max(1, Hq // Hkv // 16), bt.shape[1] * bs)[0]
+        args = (bits_to_torch(q, dev).view(torch.int16).view(dt),
+                bits_to_torch(kc, dev).view(torch.int16).view(dt),
+                bits_to_torch(vc, dev).view(torch.int16).view(dt),
+                torch.from_numpy(bt).to(dev), torch.from_numpy(ctx).to(dev), 0.09, bs)
+        base = _lib.NVJ_PHASE_SPLITK | _lib.NVJ_PHASE_COMBINE
+        a = paged_attention(*args, chunk=0, phases=base)
+        b = paged_attention(*args, chunk=0, phases=base | _lib.NVJ_PHASE_SHARED_ROWS)
+        torch.cuda.synchronize()
+        fa, fb = a.float().cpu().numpy(), b.float().cpu().numpy()
+        assert np.isfinite(fa).all()
+        assert np.abs(fa - fb).max() <= 2e-3 + 8e-3 * np.abs(fb).max(), np.abs(fa - fb).max()
+        assert not fa[ctx == 0].any()
+        if dt == torch.bfloat16:
+            assert_close_bf16(torch_to_bits(a), oracle(q, kc, vc, bt, ctx, 0.09, bs),
+                              what=f"whole rows seed={seed}")
+
+
+@pytest.mark.parametrize("B,ctx_len", [(1, 8200), (2, 6100)])
+@pytest.mark.parametrize("f16", [False, True])
+def test_balanced_split_head_dim_64_merge_in_several_passes(B, ctx_len, f16):
+    """head_dim 64: the merging wave's tile holds the (max, sum) pairs of 32 slots, so a
+    row shared by more sub-runs than that is merged in several passes (one or two long
+    sequences over all workgroups)."""
+    print(f"case D=64 several merge passes B={B} f16={f16}", flush=True)
+    import torch
+    from nanovllm_jax_amd import paged_attention
+    Hq, Hkv, D, bs = 8, 8, 64, 64
+    ctx = [ctx_len] + [ctx_len - 900] * (B - 1)
+    q, kc, vc, bt, ctx = make_problem(640 + B, B, Hq, Hkv, D, bs, sum(-(-c // bs) for c in ctx) + 1,
+                                      ctx)
+    scale = 1.0 / np.sqrt(D)
+    if not f16:
+        got = run_hip(q, kc, vc, bt, ctx, scale, bs, 0)
+        assert_close_bf16(got, oracle(q, kc, vc, bt, ctx, scale, bs), what=f"D=64 passes B={B}")
+        return
+    from oracle.paged_attention_oracle import paged_decode_attention_per_seq_ref
+    dev = "cuda:0"
+    to_f16 = lambda bits: bits_to_torch(bits, dev).float().to(torch.float16)
+    tq, tk, tv = to_f16(q), to_f16(kc), to_f16(vc)
+    out = paged_attention(tq, tk, tv, torch.from_numpy(bt).to(dev), torch.from_numpy(ctx).to(dev),
+                          scale, bs, chunk=0)
+    torch.cuda.synchronize()
+    as_bits = lambda t: t.cpu().contiguous().view(torch.int16).numpy().view(np.uint16)
+    want = paged_decode_attention_per_seq_ref(as_bits(tq), as_bits(tk), as_bits(tv), bt, ctx,
+                                              scale, bs, dtype="f16")
+    w = torch.from_numpy(want.view(np.int16)).view(torch.float16).float().numpy()
+    g = out.float().cpu().numpy()
+    assert (np.abs(g - w) <= ATOL + RTOL * np.abs(w)).all(), np.abs(g - w).max()
+
+
+def test_stale_counter_is_flagged_and_the_workspace_recovers():
+    """A counter that is not zero when a launch starts (an earlier launch cut short, two
+    launches overlapping on one workspace) loses rows; the wave that sees more arrivals
+    than the row has pieces raises the stale flag, which DecodeWorkspace.check() reads
+    back; the call after that clears the region and is right again.  Every kernel ends
+    normally."""
+    print("case stale counter flag", flush=True)
+    import torch
+    from nanovllm_jax_amd import _lib, paged_attention
+    from nanovllm_jax_amd.layers.paged_attention import DecodeWorkspace
+    B, Hq, Hkv, D, bs = 3, 32, 8, 128, 64
+    ctx = [3000, 2500, 2800]                            # every row shared by many sub-runs
+    q, kc, vc, bt, ctx = make_problem(99, B, Hq, Hkv, D, bs, sum(-(-c // bs) for c in ctx) + 1, ctx)
+    assert not deals_whole_rows(ctx, Hkv, bt.shape[1] * bs)[0]
+    dev = "cuda:0"
+    args = (bits_to_torch(q, dev), bits_to_torch(kc, dev), bits_to_torch(vc, dev),
+            torch.from_numpy(bt).to(dev), torch.from_numpy(ctx).to(dev), 0.088, bs)
+    want = oracle(q, kc, vc, bt, ctx, 0.088, bs)
+    ws = DecodeWorkspace.for_shape(B, Hq, D, bt.shape[1], bs, Hkv, dev)
+    one = _lib.NVJ_PHASE_SPLITK
+    good = paged_attention(*args, chunk=0, workspace=ws, phases=one)
+    assert ws.check()
+    assert_close_bf16(torch_to_bits(good), want, what="clean workspace")
+    ws.counters[1 + 1 * Hkv + 5] = 1000                  # (sequence 1, KV head 5)
+    bad = paged_attention(*args, chunk=0, workspace=ws, phases=one)
+    assert not ws.check(), "the stale counter went unnoticed"
+    rows = slice(5 * (Hq // Hkv), 6 * (Hq // Hkv))
+    bad_bits, good_bits = torch_to_bits(bad), torch_to_bits(good)
+    keep = np.ones(bad_bits.shape, bool)
+    keep[1, rows] = False
+    assert np.array_equal(bad_bits[keep], good_bits[keep]), "only the spoilt row may differ"
+    again = paged_attention(*args, chunk=0, workspace=ws, phases=one)   # clears first
+    assert ws.check()
+    assert np.array_equal(torch_to_bits(again), good_bits)
+    assert not ws.counters.any()
+
+
+def _hip_runtime():
+    import ctypes
+    hip = ctypes.CDLL("libamdhip64.so")
+    hip.hipMemcpy.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_size_t, ctypes.c_int]
+    hip.hipMemcpy.restype = ctypes.c_int
+    return hip
+
+
+def test_library_owned_counters_one_launch_for_any_workspace():
+    """nvj_paged_decode_launch_counters with counters = NULL: the partials in a buffer the
+    caller owns and never initialises (what an XLA custom call is handed), the counters
+    in the library's own region: bit-equal to nvj_paged_decode_launch on calls of
+    different shapes in a row; a counter of that region set from outside is flagged and
+    nvj_paged_decode_counters_reset(NULL) puts the region right again."""
+    print("case library-owned counters", flush=True)
+    import ctypes
+    import torch
+    from nanovllm_jax_amd import _lib
+    lib = _lib.load()
+    hip = _hip_runtime()
+    dev = "cuda:0"
+    stream = torch.cuda.current_stream().cuda_stream
+    region = ctypes.c_void_p()
+    size = ctypes.c_size_t()
+    assert lib.nvj_paged_decode_library_counters(ctypes.byref(region), ctypes.byref(size)) == 0
+    assert size.value == 64 << 10 and region.value
+
+    def flag():
+        torch.cuda.synchronize()
+        word = ctypes.c_int32(-1)
+        assert hip.hipMemcpy(ctypes.byref(word), region, 4, 2) == 0     # device to host
+        return word.value
+
+    def both(prob, scale, bs):
+        q, kc, vc, bt, ctx = prob
+        tq, tk, tv = (bits_to_torch(x, dev) for x in (q, kc, vc))
+        tbt, tctx = torch.from_numpy(bt).to(dev), torch.from_numpy(ctx).to(dev)
+        B, Hq, D = q.shape
+        NB, _, Hkv, _ = kc.shape
+        MB = bt.shape[1]
+        need = int(lib.nvj_paged_decode_workspace_bytes(B, Hq, D, MB, bs, Hkv, 0))
+        part = need - int(lib.nvj_paged_decode_counter_bytes(B, Hq, Hkv))
+        ws = torch.full((need,), 0xA5, dtype=torch.uint8, device=dev)
+        pt = torch.full((part,), 0x5A, dtype=torch.uint8, device=dev)
+        o1, o2 = torch.full_like(tq, 7.0), torch.full_like(tq, -7.0)
+        assert lib.nvj_paged_decode_launch(stream, tq.data_ptr(), tk.data_ptr(), tv.data_ptr(),
+                                           tbt.data_ptr(), tctx.data_ptr(), o1.data_ptr(),
+                                           ws.data_ptr(), need, B, Hq, Hkv, D, bs, MB, NB, scale,
+                                           0, 0) == 0
+        assert lib.nvj_paged_decode_launch_counters(
+            stream, tq.data_ptr(), tk.data_ptr(), tv.data_ptr(), tbt.data_ptr(), tctx.data_ptr(),
+            o2.data_ptr(), pt.data_ptr(), part, None, 0, B, Hq, Hkv, D, bs, MB, NB, scale, 0,
+            _lib.NVJ_PHASE_SPLITK) == 0
+        torch.cuda.synchronize()
+        return torch_to_bits(o1), torch_to_bits(o2)
+
+    assert lib.nvj_paged_decode_counters_reset(stream, None, 0) == 0
+    bs, D = 64, 128
+    cases = [(31, 12, 32, 8, [3000, 17, 0, 1024, 2049, 700, 1, 256, 1500, 333, 2900, 64]),
+             (32, 3, 16, 8, [700, 90, 257]),
+             (33, 40, 16, 8, [300 + 7 * i for i in range(40)])]
+    for seed, B, Hq, Hkv, ctx in cases:
+        prob = make_problem(seed, B, Hq, Hkv, D, bs, sum(-(-c // bs) for c in ctx) + 1, ctx)
+        plain, shared = both(prob, 0.088, bs)
+        assert np.array_equal(plain, shared), f"call {seed} differs"
+        assert flag() == 0
+        assert_close_bf16(shared, oracle(*prob, 0.088, bs), what=f"library counters {seed}")
+    # set one counter of the region from outside: the next call notices
+    seed, B, Hq, Hkv, ctx = cases[0]
+    prob = make_problem(seed, B, Hq, Hkv, D, bs, sum(-(-c // bs) for c in ctx) + 1, ctx)
+    bogus = ctypes.c_int32(12345)
+    assert hip.hipMemcpy(ctypes.c_void_p(region.value + 4 * (1 + 0 * Hkv + 2)),
+                         ctypes.byref(bogus), 4, 1) == 0                 # host to device
+    plain, shared = both(prob, 0.088, bs)
+    assert flag() == 1
+    assert not np.array_equal(plain, shared)
+    assert lib.nvj_paged_decode_counters_reset(stream, None, 0) == 0
+    assert flag() == 0
+    plain, shared = both(prob, 0.088, bs)
+    assert np.array_equal(plain, shared) and flag() == 0
 
 
 @pytest.mark.parametrize("B,Hkv", [(6, 8), (64, 8), (300, 4)])
@@ -313,7 +587,6 @@ def test_balanced_split_is_one_launch_that_leaves_its_counters_zero(B, Hkv):
     btt, ct = torch.from_numpy(bt).to(dev), torch.from_numpy(cap).to(dev)
     out = torch.empty_like(qt)
     ws = DecodeWorkspace.for_shape(B, Hq, D, bt.shape[1], bs, Hkv, dev)
-    counter_bytes = -(-B * Hkv * 4 // 256) * 256
     call = lambda: paged_attention(qt, kt, vt, btt, ct, 0.088, bs, chunk=0, out=out,
                                    workspace=ws, phases=_lib.NVJ_PHASE_SPLITK)
     s = torch.cuda.Stream(dev)
@@ -335,7 +608,7 @@ def test_balanced_split_is_one_launch_that_leaves_its_counters_zero(B, Hkv):
         graph.replay()
         torch.cuda.synchronize()
         replayed = torch_to_bits(out).copy()
-        assert not ws.buffer[:counter_bytes].any(), f"replay {step} left a counter set"
+        assert not ws.counters.any(), f"replay {step} left a counter set"
         eager = paged_attention(qt, kt, vt, btt, ct, 0.088, bs, chunk=0)   # fresh workspace
         torch.cuda.synchronize()
         assert np.array_equal(replayed, torch_to_bits(eager)), f"replay {step} differs from eager"
