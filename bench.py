@@ -426,8 +426,9 @@ def main():
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--workload", default="C2",
-                    choices=["C1", "C2", "C3", "C4", "C5", "R1", "C2_JITTER", "C2_SPREAD",
-                             "RAGGED_SHORT"])
+                    help="C1..C5, R1, C2_JITTER, C2_SPREAD, RAGGED_SHORT, or "
+                         "UNIFORM:<batch>:<lo>:<hi>[:<kv heads>[:<query heads>]] "
+                         "(lengths uniform in [lo, hi])")
     ap.add_argument("--shared-rows", action="store_true",
                     help="balanced split: keep the kernel from dealing whole rows to the "
                          "workgroups (the equal cut with shared rows, whatever the lengths)")

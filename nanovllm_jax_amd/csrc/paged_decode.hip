@@ -1243,7 +1243,8 @@ __global__ __launch_bounds__(512) void paged_decode_balanced_kernel(DecodeArgs a
   // whole-row layout only: the lengths of the batch where any lane can index
   // them, the order the sequences are dealt to the workgroups in, and per wave
   // the partial of a piece that has to wait for the rest of its row
-  __shared__ __align__(16) int wr_ctx[kKeptSequences];
+  __shared__ int wr_ctx[kKeptSequences];
+  __shared__ __align__(16) int wr_key[kKeptSequences];
   __shared__ int wr_order[kKeptSequences];
   __shared__ float wr_parked[NW][34 * kLanesWithDims];
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -1314,17 +1315,29 @@ __global__ __launch_bounds__(512) void paged_decode_balanced_kernel(DecodeArgs a
   // -------------------------------------------------------------------------
   if (wr_hpw > 0 && total > 0) {
     const int w_hpw = wr_hpw;
-    const int w_rps = a.num_kv_heads / w_hpw;
+    const int w_rps = a.num_kv_heads / w_hpw;       // a power of two (the host sees to it)
+    const int rps_shift = __builtin_ctz(w_rps);
     const int rows = batch * w_rps;
     const int rounds = (rows + num_wgs - 1) / num_wgs;
-    // every wave writes all the lengths itself (the same values from each),
-    // so no wave has to wait for another before it reads them back
+    // every wave writes all the lengths and step counts itself (the same values
+    // from each), so no wave has to wait for another before it reads them back
+    int longest = 0;
 #pragma unroll
-    for (int k = 0; k < kKeep; ++k) wr_ctx[k * 64 + lane] = k * 64 + lane < batch ? kept_ctx[k] : -1;
+    for (int k = 0; k < kKeep; ++k) {
+      const bool real = k * 64 + lane < batch;
+      const int n = (kept_ctx[k] + kStep - 1) / kStep;
+      wr_ctx[k * 64 + lane] = real ? kept_ctx[k] : 0;
+      // sorting key: more steps first, among equals the earlier sequence first;
+      // unique, and below every real key for the padding behind the batch
+      wr_key[k * 64 + lane] = real ? (n << 8) | (255 - (k * 64 + lane)) : -1 - (k * 64 + lane);
+      longest = max(longest, n);
+    }
+#pragma unroll
+    for (int m = 32; m >= 1; m >>= 1) longest = max(longest, __shfl_xor(longest, m, 64));
+    longest = __builtin_amdgcn_readfirstlane(longest);
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
     __builtin_amdgcn_wave_barrier();
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-    auto steps_at = [&](int seq) { return (wr_ctx[seq] + kStep - 1) / kStep; };
     // the largest number of steps any workgroup is dealt, `sorted`: through wr_order
     auto largest_deal = [&](bool sorted) {
       int worst = 0;
@@ -1334,8 +1347,8 @@ __global__ __launch_bounds__(512) void paged_decode_balanced_kernel(DecodeArgs a
         for (int t = 0; t < rounds; ++t) {
           const int p = t * num_wgs + ((t & 1) ? num_wgs - 1 - w : w);
           if (w < num_wgs && p < rows) {
-            const int rank = p / w_rps;
-            load += steps_at(sorted ? wr_order[rank] : rank);
+            const int rank = p >> rps_shift;
+            load += wr_key[sorted ? wr_order[rank] : rank] >> 8;
           }
         }
         worst = max(worst, load);
@@ -1345,30 +1358,27 @@ __global__ __launch_bounds__(512) void paged_decode_balanced_kernel(DecodeArgs a
       return __builtin_amdgcn_readfirstlane(worst);
     };
     const int64_t budget = (int64_t)w_rps * total * (256 + wr_tol);   // 256 * num_wgs * the limit
-    bool whole_rows = (int64_t)largest_deal(false) * num_wgs * 256 <= budget;
+    const auto fits = [&](int load) { return (int64_t)load * num_wgs * 256 <= budget; };
+    // a row longer than the limit rules both orders out
+    // (with one round every workgroup gets one row, and the longest row decides)
+    bool whole_rows = fits(longest) && (rounds == 1 || fits(largest_deal(false)));
     bool sorted = false;
-    if (!whole_rows && rounds > 1) {
-      // rank of every sequence by decreasing number of steps, ties in batch
-      // order: two threads per sequence count, over half of the batch each,
-      // the sequences that come before it
+    if (!whole_rows && rounds > 1 && fits(longest)) {
+      // rank of every sequence by decreasing key: two threads per sequence
+      // count, over half of the batch each, the keys above its own
       const int i = threadIdx.x >> 1, half = threadIdx.x & 1;
-      const int ni = i < batch ? steps_at(i) : -1;
-      int before = 0;
+      const int mine = wr_key[i];
+      int above = 0;
       for (int j4 = half * (kKeptSequences / 8); j4 < (half + 1) * (kKeptSequences / 8); ++j4) {
-        const int4 c4 = reinterpret_cast<const int4*>(wr_ctx)[j4];
-        const int cj[4] = {c4.x, c4.y, c4.z, c4.w};
-#pragma unroll
-        for (int u = 0; u < 4; ++u) {
-          const int j = 4 * j4 + u;
-          const int nj = cj[u] < 0 ? -1 : (cj[u] + kStep - 1) / kStep;
-          before += (nj > ni || (nj == ni && j < i)) ? 1 : 0;
-        }
+        const int4 k4 = reinterpret_cast<const int4*>(wr_key)[j4];
+        above += (k4.x > mine ? 1 : 0) + (k4.y > mine ? 1 : 0) + (k4.z > mine ? 1 : 0) +
+                 (k4.w > mine ? 1 : 0);
       }
-      before += __builtin_amdgcn_update_dpp(0, before, kDppQuadXor1, 0xF, 0xF, false);
-      if (half == 0) wr_order[before] = i;
+      above += __builtin_amdgcn_update_dpp(0, above, kDppQuadXor1, 0xF, 0xF, false);
+      if (half == 0) wr_order[above] = i;
       __syncthreads();
       sorted = true;
-      whole_rows = (int64_t)largest_deal(true) * num_wgs * 256 <= budget;
+      whole_rows = fits(largest_deal(true));
     }
     if (whole_rows) {
       const int w_parts = NW / w_hpw;
@@ -1817,7 +1827,8 @@ bool plan_workspace(int64_t batch, int64_t num_heads, int64_t head_dim, int64_t 
     if (batch <= kKeptSequences)
       for (int h = hpw; h >= 2; h /= 2)
         if (num_kv_heads % h == 0 && batch * (num_kv_heads / h) >= wgs) {
-          plan->wr_hpw = h;
+          const int rps = num_kv_heads / h;
+          if ((rps & (rps - 1)) == 0) plan->wr_hpw = h;   // the kernel divides by shifting
           break;
         }
     plan->max_chunks = 0;

@@ -141,6 +141,22 @@ def make_workload(name: str, seed: int | None = None) -> DecodeWorkload:
         MB = int(nblk.max())
         bt = _tables_from_counts(rng, nblk, NB, MB)
         gain = 1.0
+    elif name.startswith("UNIFORM:"):
+        # UNIFORM:<batch>:<lo>:<hi>[:<kv heads>[:<query heads>]]: lengths uniform in
+        # [lo, hi], Qwen3-8B heads unless given; a measuring aid (bench.py --workload)
+        f = [int(x) for x in name.split(":")[1:]]
+        B, lo, hi = f[0], f[1], f[2]
+        Hkv = f[3] if len(f) > 3 else 8
+        Hq = f[4] if len(f) > 4 else 4 * Hkv
+        D, bs = 128, 256
+        seed = 2000 + B if seed is None else seed
+        rng = np.random.Generator(np.random.PCG64(seed))
+        ctx = rng.integers(lo, hi + 1, size=B).astype(np.int32)
+        nblk = -(-ctx // bs)
+        NB = int(np.ceil(1.1 * nblk.sum())) + 1
+        MB = max(int(nblk.max()), 1)
+        bt = _tables_from_counts(rng, nblk, NB, MB)
+        gain = 1.0
     else:
         raise KeyError(name)
     return DecodeWorkload(name=name, batch=B, num_heads=Hq, num_kv_heads=Hkv,

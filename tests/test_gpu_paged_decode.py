@@ -278,7 +278,8 @@ def deals_whole_rows(ctx, num_kv_heads, table_positions, cus=256, tolerance=16):
     h = hpw
     while B <= 256 and h >= 2:
         if num_kv_heads % h == 0 and B * (num_kv_heads // h) >= wgs:
-            wr = h
+            rps = num_kv_heads // h
+            wr = h if rps & (rps - 1) == 0 else 0      # rows per sequence: a power of two
             break
         h //= 2
     steps = _steps(ctx, table_positions)
