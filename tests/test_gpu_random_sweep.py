@@ -70,12 +70,14 @@ def _prefill_case(rng):
     return dict(Hq=Hkv * G, Hkv=Hkv, lens_q=lens_q, lens_k=lens_k, scale=scale, gain=gain)
 
 
-@pytest.mark.parametrize("seed", range(24))
-def test_prefill_random_case(seed):
+def _run_prefill_case(seed):
+    """Case `seed` of the prefill generator through the HIP kernel: the output bits, the
+    bf16-probability oracle's, and the exact float64 softmax."""
     import torch
     from nanovllm_jax_amd import variable_length_attention_prefill
     from nanovllm_jax_amd.workloads import draw_bf16_bits
-    from oracle.paged_attention_oracle import variable_length_attention_prefill_ref
+    from oracle.paged_attention_oracle import (textbook_prefill_f64,
+                                               variable_length_attention_prefill_ref)
     c = _prefill_case(np.random.Generator(np.random.PCG64(41000 + seed)))
     print(f"case prefill sweep seed={seed} {c}", flush=True)
     rng = np.random.Generator(np.random.PCG64(42000 + seed))
@@ -89,19 +91,51 @@ def test_prefill_random_case(seed):
         bits_to_torch(q, dev), bits_to_torch(k, dev), bits_to_torch(v, dev),
         torch.from_numpy(cu_q).to(dev), torch.from_numpy(cu_k).to(dev), scale=c["scale"])
     torch.cuda.synchronize()
-    got = torch_to_bits(out)
     want = variable_length_attention_prefill_ref(q, k, v, cu_q, cu_k, c["scale"])
+    exact = np.asarray(textbook_prefill_f64(q, k, v, cu_q, cu_k, c["scale"]), np.float64)
+    return torch_to_bits(out), want, exact
+
+
+def _excess_over_the_bar(got_bits, want):
+    """How far the worst element lies outside atol/rtol 1e-2 of `want` (<= 0: inside)."""
+    from oracle.paged_attention_oracle import bf16_bits_to_f32
+    got = bf16_bits_to_f32(got_bits).astype(np.float64)
+    want = np.asarray(want, np.float64)
+    return float((np.abs(got - want) - (1e-2 + 1e-2 * np.abs(want))).max())
+
+
+@pytest.mark.parametrize("seed", range(24))
+def test_prefill_random_case(seed):
+    from oracle.paged_attention_oracle import bf16_bits_to_f32
+    got, want, exact = _run_prefill_case(seed)
     assert_close_bf16(got, want, what=f"prefill sweep seed={seed}")
     # Also against the exact float64 softmax.  The oracle above rounds the
     # probabilities to bf16 as the reference's attention does, the kernel rounds
-    # its own (differently scaled) ones: two independent roundings.  Over 2000
-    # further seeds of this generator five cases had one element outside the bar
-    # against that oracle, by at most 1.3e-3, while the kernel itself stayed at
-    # least 2.6e-3 inside it against float64; this is the check for the kernel.
-    from oracle.paged_attention_oracle import bf16_bits_to_f32, textbook_prefill_f64
-    exact = np.asarray(textbook_prefill_f64(q, k, v, cu_q, cu_k, c["scale"]), np.float64)
-    err = np.abs(bf16_bits_to_f32(got).astype(np.float64) - exact)
-    assert np.all(err <= 1e-2 + 1e-2 * np.abs(exact)), f"seed={seed}: max err {err.max():.3e} vs float64"
+    # its own (differently scaled) ones: two independent roundings.
+    assert _excess_over_the_bar(got, exact) <= 0, f"seed={seed} vs float64"
+
+
+@pytest.mark.parametrize("seed", [871, 1316, 1393, 1448, 1753])
+def test_prefill_cases_at_the_edge_of_the_bar(seed):
+    """The five cases of a 2000-seed run of the same generator in which one output
+    element lay outside the bar against the bf16-probability oracle (by up to 1.3e-3)
+    while inside it against float64.  The oracle normalises the probabilities and then
+    rounds them to bf16 (the reference's dot_product_attention); the kernel rounds
+    unnormalised ones and divides by the sum of the rounded values, so that a row with
+    one dominant key reproduces that key's V exactly: two roundings of different numbers,
+    each within the bar of the exact result, up to 2^-8 apart from each other.  The
+    assertion is the float64 one; the distance to the oracle's bar is printed and
+    bounded, so that a kernel change that widens it is seen."""
+    from oracle.paged_attention_oracle import bf16_bits_to_f32
+    got, want, exact = _run_prefill_case(seed)
+    vs_exact = _excess_over_the_bar(got, exact)
+    vs_oracle = _excess_over_the_bar(got, bf16_bits_to_f32(want))
+    oracle_vs_exact = _excess_over_the_bar(want, exact)
+    print(f"  seed {seed}: kernel vs float64 {vs_exact:+.2e}, kernel vs bf16-probability oracle "
+          f"{vs_oracle:+.2e}, that oracle vs float64 {oracle_vs_exact:+.2e} "
+          "(distance of the worst element to the bar, negative = inside)", flush=True)
+    assert vs_exact <= -2e-3, f"seed={seed}: the kernel itself is at the edge of the bar"
+    assert vs_oracle <= 2e-3, f"seed={seed}: further outside the oracle's bar than measured before"
 
 
 def _paged_prefill_case(rng):
