@@ -94,11 +94,13 @@ NVJ_API int nvj_store_kvcache_launch(void* stream,
  *               context_lens on the device and lays the work out itself, so
  *               ragged batches are balanced without the host knowing the
  *               lengths.  Where whole (sequence, head group) rows can be dealt
- *               to the workgroups within 1/16 of an equal share of the
+ *               to the workgroups within a quarter of an equal share of the
  *               32-position steps (lengths equal or nearly so; or, taken by
  *               decreasing length, long rows that pair up with short ones), no
  *               row is shared between workgroups and the workspace is not
- *               touched.  Otherwise the steps of all rows, end to end, are cut
+ *               touched (the launch is bound by the memory system as a whole,
+ *               so an uneven deal costs far less than its unevenness, and
+ *               less than sharing rows does).  Otherwise the steps of all rows, end to end, are cut
  *               into equal runs, one per wave; a row that fits one workgroup is
  *               finished there, a row shared by several is merged by the wave
  *               that completes it (counters in the workspace), without a

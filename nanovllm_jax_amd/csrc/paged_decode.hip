@@ -952,6 +952,11 @@ __device__ __forceinline__ int wave_inclusive_scan(int x) {
 // after its one pass over the lengths; further ones are read again when needed.
 constexpr int kKeptSequences = 256;
 
+// Whole rows in the order of the batch, several rows per workgroup: only when
+// no workgroup gets more than 1 + 8/256 of the mean (beyond that the order by
+// length, which the caller's tolerance applies to, usually does better).
+constexpr int kWholeRowTightTolerance = 8;
+
 // The cut of the axis: sub-run j covers the axis positions whose unit
 // (position >> shift) lies in [floor(j * units / nsub), floor((j+1) * units / nsub)).
 // shift is 0 unless the axis is so long that units * nsub would not fit 31 bits
@@ -1361,7 +1366,12 @@ __global__ __launch_bounds__(512) void paged_decode_balanced_kernel(DecodeArgs a
     const auto fits = [&](int load) { return (int64_t)load * num_wgs * 256 <= budget; };
     // a row longer than the limit rules both orders out
     // (with one round every workgroup gets one row, and the longest row decides)
-    bool whole_rows = fits(longest) && (rounds == 1 || fits(largest_deal(false)));
+    // (with more rounds the order of the batch is only taken when it is as good
+    // as balanced; otherwise the order by length gets its chance first)
+    bool whole_rows =
+        fits(longest) &&
+        (rounds == 1 || (int64_t)largest_deal(false) * num_wgs * 256 <=
+                            (int64_t)w_rps * total * (256 + min(wr_tol, kWholeRowTightTolerance)));
     bool sorted = false;
     if (!whole_rows && rounds > 1 && fits(longest)) {
       // rank of every sequence by decreasing key: two threads per sequence
@@ -1774,8 +1784,15 @@ int balanced_heads_per_workgroup(int64_t batch, int num_kv_heads, int64_t max_st
 constexpr int kMinBalancedSteps = 1;
 
 // Whole rows are dealt to the workgroups when no workgroup gets more than
-// 1 + kWholeRowTolerance / 256 times the mean number of steps.
-constexpr int kWholeRowTolerance = 16;
+// 1 + kWholeRowTolerance / 256 times the mean number of steps.  The launch is
+// bound by the memory system as a whole, not by its slowest workgroup: while
+// workgroups with less to do finish, the others stream faster, so an uneven
+// deal costs far less than its unevenness.  Measured against the equal cut with
+// shared rows (256 sequences, 2 rows each, lengths log-uniform or uniform):
+// 9 % unevenness 195 against 213 us, 16 % 174 against 187, 34 % 148 against
+// 149, 56 % 250 against 231; one row per workgroup (64 sequences around 3500
+// positions): 9 % 153 against 165, 15 % 146 against 154, 25 % 137 against 142.
+constexpr int kWholeRowTolerance = 64;
 
 // Waves per workgroup of the fixed split = KV heads a workgroup covers: the
 // largest of 8, 4, 2, 1 that divides the number of KV heads.

@@ -141,9 +141,10 @@ def make_workload(name: str, seed: int | None = None) -> DecodeWorkload:
         MB = int(nblk.max())
         bt = _tables_from_counts(rng, nblk, NB, MB)
         gain = 1.0
-    elif name.startswith("UNIFORM:"):
+    elif name.startswith("UNIFORM:") or name.startswith("LOGUNIFORM:"):
         # UNIFORM:<batch>:<lo>:<hi>[:<kv heads>[:<query heads>]]: lengths uniform in
-        # [lo, hi], Qwen3-8B heads unless given; a measuring aid (bench.py --workload)
+        # [lo, hi] (LOGUNIFORM: their logarithms are), Qwen3-8B heads unless given; a
+        # measuring aid (bench.py --workload)
         f = [int(x) for x in name.split(":")[1:]]
         B, lo, hi = f[0], f[1], f[2]
         Hkv = f[3] if len(f) > 3 else 8
@@ -151,7 +152,10 @@ def make_workload(name: str, seed: int | None = None) -> DecodeWorkload:
         D, bs = 128, 256
         seed = 2000 + B if seed is None else seed
         rng = np.random.Generator(np.random.PCG64(seed))
-        ctx = rng.integers(lo, hi + 1, size=B).astype(np.int32)
+        if name.startswith("LOG"):
+            ctx = np.rint(np.exp(rng.uniform(np.log(lo), np.log(hi), size=B))).astype(np.int32)
+        else:
+            ctx = rng.integers(lo, hi + 1, size=B).astype(np.int32)
         nblk = -(-ctx // bs)
         NB = int(np.ceil(1.1 * nblk.sum())) + 1
         MB = max(int(nblk.max()), 1)

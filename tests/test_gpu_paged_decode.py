@@ -258,7 +258,7 @@ def _steps(ctx, cap):
     return -(-np.clip(np.asarray(ctx, np.int64), 0, cap) // 32)
 
 
-def deals_whole_rows(ctx, num_kv_heads, table_positions, cus=256, tolerance=16):
+def deals_whole_rows(ctx, num_kv_heads, table_positions, cus=256, tolerance=64, tight=8):
     """The balanced kernel's own layout rule, restated: are whole (sequence, head
     group) rows dealt to the workgroups (nothing shared, workspace untouched)?
     Returns (whole_rows, sorted): `sorted` when it took the order by decreasing
@@ -297,7 +297,11 @@ def deals_whole_rows(ctx, num_kv_heads, table_positions, cus=256, tolerance=16):
         return int(load.max())
 
     budget = rps * int(steps.sum()) * (256 + tolerance)
-    if largest(np.arange(B)) * wgs * 256 <= budget:
+    if int(steps.max()) * wgs * 256 > budget:          # one row alone is too much
+        return False, False
+    # the order of the batch: with several rows per workgroup only when all but even
+    first = budget if rounds == 1 else rps * int(steps.sum()) * (256 + min(tolerance, tight))
+    if largest(np.arange(B)) * wgs * 256 <= first:
         return True, False
     if rounds > 1 and largest(np.argsort(-steps, kind="stable")) * wgs * 256 <= budget:
         return True, True
@@ -326,26 +330,31 @@ def _run_over_marked_workspace(q, kc, vc, bt, ctx, scale, bs, extra_phases=0):
 
 
 @pytest.mark.parametrize("name", ["equal", "within_tolerance", "one_short", "one_long",
+                                  "a_sixth_apart", "a_half_apart",
                                   "pairs_by_length", "pairs_four_rounds", "log_uniform",
                                   "equal_forced_shared"])
 def test_balanced_split_deals_whole_rows_when_that_is_balanced(name):
     """The kernel looks at the lengths and, when whole rows can be dealt to the
-    workgroups within 1/16 of an equal share, shares no row (the workspace stays
-    untouched): equal lengths; lengths a few percent apart; one short sequence among
-    equal ones; lengths that only balance when long rows are paired with short ones
+    workgroups within a quarter of an equal share, shares no row (the workspace stays
+    untouched): equal lengths; lengths a few percent or a sixth apart; one short
+    sequence among equal ones; lengths that only balance when long rows are paired with short ones
     (the order by decreasing length, two and four rounds of rows).  It must not do so
-    when one long sequence or a log-uniform spread would leave workgroups idle, and
+    when one long sequence, lengths a half apart or a log-uniform spread would leave
+    workgroups idle for long, and
     not when the caller forbids it.  Every case against the oracle, and the layout
     against the rule restated in deals_whole_rows."""
     print(f"case whole rows {name}", flush=True)
     from nanovllm_jax_amd import _lib
     rng = np.random.Generator(np.random.PCG64(len(name) * 131 + 5))
     bs, extra = 64, 0
-    if name in ("equal", "equal_forced_shared", "within_tolerance", "one_short", "one_long"):
+    if name in ("equal", "equal_forced_shared", "within_tolerance", "one_short", "one_long",
+                "a_sixth_apart", "a_half_apart"):
         B, Hq, Hkv, D = 128, 8, 4, 128                 # 128 rows of 4 heads, 256 rows of 2
         ctx = {"equal": lambda: rng.integers(930, 961, size=B),            # 30 steps each
                "equal_forced_shared": lambda: rng.integers(930, 961, size=B),
                "within_tolerance": lambda: rng.integers(870, 961, size=B),  # 28..30 steps
+               "a_sixth_apart": lambda: rng.integers(700, 961, size=B),     # 22..30 steps
+               "a_half_apart": lambda: rng.integers(300, 961, size=B),      # 10..30 steps
                "one_short": lambda: np.where(np.arange(B) == 77, 100, 960),
                "one_long": lambda: np.where(np.arange(B) == 77, 2900, 960)}[name]()
         if name == "equal_forced_shared":
@@ -367,6 +376,7 @@ def test_balanced_split_deals_whole_rows_when_that_is_balanced(name):
     whole, by_length = deals_whole_rows(ctx, Hkv, bt.shape[1] * bs)
     expect = {"equal": (True, False), "within_tolerance": (True, False),
               "one_short": (True, False), "one_long": (False, False),
+              "a_sixth_apart": (True, False), "a_half_apart": (False, False),
               "pairs_by_length": (True, True), "pairs_four_rounds": (True, True),
               "log_uniform": (False, False), "equal_forced_shared": (True, False)}[name]
     assert (whole, by_length) == expect, "the case does not exercise what its name says"
