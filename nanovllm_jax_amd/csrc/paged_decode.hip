@@ -915,6 +915,18 @@ __device__ __forceinline__ int wave_inclusive_scan(int x) {
   return x;
 }
 
+// Maximum over the 64 lanes of a wave, wave-uniform, with the same DPP moves (a
+// lane without a source keeps its own value).
+__device__ __forceinline__ int wave_max(int x) {
+  x = max(x, __builtin_amdgcn_update_dpp(x, x, 0x111, 0xF, 0xF, false));
+  x = max(x, __builtin_amdgcn_update_dpp(x, x, 0x112, 0xF, 0xF, false));
+  x = max(x, __builtin_amdgcn_update_dpp(x, x, 0x114, 0xF, 0xF, false));
+  x = max(x, __builtin_amdgcn_update_dpp(x, x, 0x118, 0xF, 0xF, false));
+  x = max(x, __builtin_amdgcn_update_dpp(x, x, 0x142, 0xA, 0xF, false));
+  x = max(x, __builtin_amdgcn_update_dpp(x, x, 0x143, 0xC, 0xF, false));
+  return __builtin_amdgcn_readlane(x, 63);
+}
+
 // ---------------------------------------------------------------------------
 // Balanced split: one launch for any mix of lengths.
 //
@@ -1249,8 +1261,10 @@ __global__ __launch_bounds__(512) void paged_decode_balanced_kernel(DecodeArgs a
   // them, the order the sequences are dealt to the workgroups in, and per wave
   // the partial of a piece that has to wait for the rest of its row
   __shared__ int wr_ctx[kKeptSequences];
-  __shared__ __align__(16) int wr_key[kKeptSequences];
-  __shared__ int wr_order[kKeptSequences];
+  __shared__ int wr_steps[kKeptSequences];    // steps of every sequence
+  __shared__ __align__(16) int wr_key[kKeptSequences];   // sorting keys
+  __shared__ int wr_order[kKeptSequences];    // sequence of every rank by length
+  __shared__ int wr_sorted[kKeptSequences];   // its steps
   __shared__ float wr_parked[NW][34 * kLanesWithDims];
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int lane = threadIdx.x & 63;
@@ -1326,69 +1340,91 @@ __global__ __launch_bounds__(512) void paged_decode_balanced_kernel(DecodeArgs a
     const int rounds = (rows + num_wgs - 1) / num_wgs;
     // every wave writes all the lengths and step counts itself (the same values
     // from each), so no wave has to wait for another before it reads them back
-    int longest = 0;
+    int key[kKeep];
+    int longest = 0, shortest = INT32_MAX;
 #pragma unroll
     for (int k = 0; k < kKeep; ++k) {
       const bool real = k * 64 + lane < batch;
       const int n = (kept_ctx[k] + kStep - 1) / kStep;
       wr_ctx[k * 64 + lane] = real ? kept_ctx[k] : 0;
+      wr_steps[k * 64 + lane] = real ? n : 0;
       // sorting key: more steps first, among equals the earlier sequence first;
       // unique, and below every real key for the padding behind the batch
-      wr_key[k * 64 + lane] = real ? (n << 8) | (255 - (k * 64 + lane)) : -1 - (k * 64 + lane);
-      longest = max(longest, n);
+      key[k] = real ? (n << 8) | (255 - (k * 64 + lane)) : -1 - (k * 64 + lane);
+      longest = max(longest, real ? n : 0);
+      shortest = min(shortest, real ? n : INT32_MAX);
     }
-#pragma unroll
-    for (int m = 32; m >= 1; m >>= 1) longest = max(longest, __shfl_xor(longest, m, 64));
-    longest = __builtin_amdgcn_readfirstlane(longest);
+    longest = wave_max(longest);
+    shortest = -wave_max(-shortest);
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
     __builtin_amdgcn_wave_barrier();
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-    // the largest number of steps any workgroup is dealt, `sorted`: through wr_order
-    auto largest_deal = [&](bool sorted) {
+    // the largest number of steps any workgroup is dealt; steps_of_rank: the
+    // steps of the sequence of a given rank (wr_steps in the order of the batch,
+    // wr_sorted in the order by length)
+    auto largest_deal = [&](const int* steps_of_rank) {
       int worst = 0;
-      for (int w0 = 0; w0 < num_wgs; w0 += 64) {
+#pragma unroll
+      for (int w0 = 0; w0 < 256; w0 += 64) {    // the whole-row layout is offered up to 256 workgroups
         const int w = w0 + lane;
         int load = 0;
         for (int t = 0; t < rounds; ++t) {
           const int p = t * num_wgs + ((t & 1) ? num_wgs - 1 - w : w);
-          if (w < num_wgs && p < rows) {
-            const int rank = p >> rps_shift;
-            load += wr_key[sorted ? wr_order[rank] : rank] >> 8;
-          }
+          if (w < num_wgs && p < rows) load += steps_of_rank[p >> rps_shift];
         }
         worst = max(worst, load);
       }
-#pragma unroll
-      for (int m = 32; m >= 1; m >>= 1) worst = max(worst, __shfl_xor(worst, m, 64));
-      return __builtin_amdgcn_readfirstlane(worst);
+      return wave_max(worst);
     };
     const int64_t budget = (int64_t)w_rps * total * (256 + wr_tol);   // 256 * num_wgs * the limit
     const auto fits = [&](int load) { return (int64_t)load * num_wgs * 256 <= budget; };
-    // a row longer than the limit rules both orders out
-    // (with one round every workgroup gets one row, and the longest row decides)
-    // (with more rounds the order of the batch is only taken when it is as good
-    // as balanced; otherwise the order by length gets its chance first)
-    bool whole_rows =
-        fits(longest) &&
-        (rounds == 1 || (int64_t)largest_deal(false) * num_wgs * 256 <=
-                            (int64_t)w_rps * total * (256 + min(wr_tol, kWholeRowTightTolerance)));
+    // A row longer than the limit rules both orders out.  With one round every
+    // workgroup gets one row and the longest row decides.  With more rounds the
+    // order of the batch is only taken when it is as good as balanced (and only
+    // looked at when the lengths are within an eighth of each other); otherwise
+    // the order by length gets its chance.
+    bool whole_rows = fits(longest);
     bool sorted = false;
-    if (!whole_rows && rounds > 1 && fits(longest)) {
-      // rank of every sequence by decreasing key: two threads per sequence
-      // count, over half of the batch each, the keys above its own
-      const int i = threadIdx.x >> 1, half = threadIdx.x & 1;
-      const int mine = wr_key[i];
-      int above = 0;
-      for (int j4 = half * (kKeptSequences / 8); j4 < (half + 1) * (kKeptSequences / 8); ++j4) {
-        const int4 k4 = reinterpret_cast<const int4*>(wr_key)[j4];
-        above += (k4.x > mine ? 1 : 0) + (k4.y > mine ? 1 : 0) + (k4.z > mine ? 1 : 0) +
-                 (k4.w > mine ? 1 : 0);
+    if (whole_rows && rounds > 1) {
+      whole_rows = (longest - shortest) * 8 <= longest &&
+                   (int64_t)largest_deal(wr_steps) * num_wgs * 256 <=
+                       (int64_t)w_rps * total * (256 + min(wr_tol, kWholeRowTightTolerance));
+      if (!whole_rows) {
+        // Rank of every sequence by decreasing key: two threads per sequence
+        // count, over half of the batch each, the keys above its own.  The keys
+        // go through LDS (every wave writes all of them, the same values from
+        // each) and are read back four at a time, eight reads in flight.
+#pragma unroll
+        for (int k = 0; k < kKeep; ++k) wr_key[k * 64 + lane] = key[k];
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+        const int i = threadIdx.x >> 1, half = threadIdx.x & 1;
+        const int mine = wr_key[i];
+        const int quads = (batch + 3) / 4;            // int4 groups that hold real keys
+        const int per_half = (quads + 1) / 2;
+        int above = 0;
+        for (int j0 = half * per_half; j0 < min(quads, (half + 1) * per_half); j0 += 8) {
+          int4 k4[8];
+#pragma unroll
+          for (int u = 0; u < 8; ++u)
+            k4[u] = reinterpret_cast<const int4*>(wr_key)[min(j0 + u, kKeptSequences / 4 - 1)];
+#pragma unroll
+          for (int u = 0; u < 8; ++u) {
+            const bool in = j0 + u < min(quads, (half + 1) * per_half);
+            above += (in && k4[u].x > mine ? 1 : 0) + (in && k4[u].y > mine ? 1 : 0) +
+                     (in && k4[u].z > mine ? 1 : 0) + (in && k4[u].w > mine ? 1 : 0);
+          }
+        }
+        above += __builtin_amdgcn_update_dpp(0, above, kDppQuadXor1, 0xF, 0xF, false);
+        if (half == 0 && i < batch) {
+          wr_order[above] = i;
+          wr_sorted[above] = mine >> 8;
+        }
+        __syncthreads();
+        sorted = true;
+        whole_rows = fits(largest_deal(wr_sorted));
       }
-      above += __builtin_amdgcn_update_dpp(0, above, kDppQuadXor1, 0xF, 0xF, false);
-      if (half == 0) wr_order[above] = i;
-      __syncthreads();
-      sorted = true;
-      whole_rows = fits(largest_deal(true));
     }
     if (whole_rows) {
       const int w_parts = NW / w_hpw;
