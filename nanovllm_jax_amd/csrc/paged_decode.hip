@@ -26,7 +26,8 @@
 //   * V: 8 x 16-byte loads per lane straight from HBM, one per position the
 //     lane's P^T operand holds, transposed inside the lane with v_perm_b32
 //     into 8 A operands (lane = 8 dims x 8 positions), so no LDS for V.
-//   * O^T[dim, qhead] += V^T . P^T with 8 MFMAs.
+//   * O^T[dim, qhead] += V^T . P^T with 16 MFMAs: P enters twice, as its values
+//     rounded to the cache's 16-bit type and as the rest of that rounding.
 // Loads for step i+1 are issued before the arithmetic of step i.
 //
 // In the first two modes the partial (unnormalised O, running max, running
@@ -77,6 +78,13 @@ template <> struct Elem<false> {
     bf16x2 p = {(__bf16)lo, (__bf16)hi};
     return __builtin_bit_cast(uint32_t, p);
   }
+  // the two values a packed pair stands for
+  static __device__ __forceinline__ float low_of(uint32_t pair) {
+    return __builtin_bit_cast(float, pair << 16);
+  }
+  static __device__ __forceinline__ float high_of(uint32_t pair) {
+    return __builtin_bit_cast(float, pair & 0xFFFF0000u);
+  }
 };
 template <> struct Elem<true> {
   static __device__ __forceinline__ f32x4 mfma(uint4 a, uint4 b, f32x4 c) {
@@ -88,7 +96,24 @@ template <> struct Elem<true> {
     f16x2 p = {(_Float16)lo, (_Float16)hi};   // round to nearest even
     return __builtin_bit_cast(uint32_t, p);
   }
+  static __device__ __forceinline__ float low_of(uint32_t pair) {
+    typedef __attribute__((ext_vector_type(2))) _Float16 f16x2;
+    return (float)__builtin_bit_cast(f16x2, pair)[0];
+  }
+  static __device__ __forceinline__ float high_of(uint32_t pair) {
+    typedef __attribute__((ext_vector_type(2))) _Float16 f16x2;
+    return (float)__builtin_bit_cast(f16x2, pair)[1];
+  }
 };
+
+// A pair of fp32 values as two packed pairs of the cache's 16-bit type: the
+// rounded values and what the rounding left over, rounded again.  Their sum
+// carries 16 (bf16) or 22 (float16) mantissa bits of the fp32 values.
+template <bool F16>
+__device__ __forceinline__ void pack2_with_rest(float a, float b, uint32_t& main, uint32_t& rest) {
+  main = Elem<F16>::pack2(a, b);
+  rest = Elem<F16>::pack2(a - Elem<F16>::low_of(main), b - Elem<F16>::high_of(main));
+}
 
 
 __device__ __forceinline__ float wave_xor_max(float x, int mask) {
@@ -321,11 +346,16 @@ __device__ __forceinline__ void compute_segment(const DecodeArgs& a, uint4* lds,
 #pragma unroll
     for (int e = 0; e < 4; ++e) psum += p0[e] + p1[e];
     l_run = fmaf(l_run, alpha, psum);
-    uint4 pbits;
-    pbits.x = Elem<F16>::pack2(p0[0], p0[1]);
-    pbits.y = Elem<F16>::pack2(p0[2], p0[3]);
-    pbits.z = Elem<F16>::pack2(p1[0], p1[1]);
-    pbits.w = Elem<F16>::pack2(p1[2], p1[3]);
+    // The probabilities go to the matrix core as two operands of the cache's
+    // 16-bit type, the rounded values and the rest of the rounding, so that
+    // P.V sees them to 16 bits or more, as good as the fp32 probabilities of the
+    // reference's vectorised path (layers/pallas_attention.py:227-236); the
+    // second product is free under the K/V stream.
+    uint4 pbits, prest;
+    pack2_with_rest<F16>(p0[0], p0[1], pbits.x, prest.x);
+    pack2_with_rest<F16>(p0[2], p0[3], pbits.y, prest.y);
+    pack2_with_rest<F16>(p1[0], p1[1], pbits.z, prest.z);
+    pack2_with_rest<F16>(p1[2], p1[3], pbits.w, prest.w);
 
     // ---- V: in-lane 8x8 transpose (positions x dims), then next V loads ----
     uint4 vt[8];
@@ -357,6 +387,7 @@ __device__ __forceinline__ void compute_segment(const DecodeArgs& a, uint4* lds,
     for (int jd = 0; jd < 8; ++jd) {
       acc[jd] *= alpha;
       acc[jd] = Elem<F16>::mfma(vt[jd], pbits, acc[jd]);
+      acc[jd] = Elem<F16>::mfma(vt[jd], prest, acc[jd]);
     }
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
     __builtin_amdgcn_wave_barrier();
@@ -968,6 +999,9 @@ constexpr int kKeptSequences = 256;
 // no workgroup gets more than 1 + 8/256 of the mean (beyond that the order by
 // length, which the caller's tolerance applies to, usually does better).
 constexpr int kWholeRowTightTolerance = 8;
+// The whole-row layout is offered for launches of up to this many workgroups
+// (every wave checks the deal of all of them, 64 per pass).
+constexpr int kMaxWholeRowWorkgroups = 256;
 
 // The cut of the axis: sub-run j covers the axis positions whose unit
 // (position >> shift) lies in [floor(j * units / nsub), floor((j+1) * units / nsub)).
@@ -1365,7 +1399,7 @@ __global__ __launch_bounds__(512) void paged_decode_balanced_kernel(DecodeArgs a
     auto largest_deal = [&](const int* steps_of_rank) {
       int worst = 0;
 #pragma unroll
-      for (int w0 = 0; w0 < 256; w0 += 64) {    // the whole-row layout is offered up to 256 workgroups
+      for (int w0 = 0; w0 < kMaxWholeRowWorkgroups; w0 += 64) {
         const int w = w0 + lane;
         int load = 0;
         for (int t = 0; t < rounds; ++t) {
@@ -1877,7 +1911,7 @@ bool plan_workspace(int64_t batch, int64_t num_heads, int64_t head_dim, int64_t 
     // least: with 1 the K/V stream of a large launch is a tenth slower).  It
     // needs no workspace of its own.
     plan->wr_hpw = 0;
-    if (batch <= kKeptSequences)
+    if (batch <= kKeptSequences && wgs <= kMaxWholeRowWorkgroups)
       for (int h = hpw; h >= 2; h /= 2)
         if (num_kv_heads % h == 0 && batch * (num_kv_heads / h) >= wgs) {
           const int rps = num_kv_heads / h;
