@@ -386,8 +386,9 @@ def test_balanced_split_deals_whole_rows_when_that_is_balanced(name):
 
 def test_balanced_split_whole_rows_equal_the_shared_rows_split():
     """The two layouts of chunk = 0 on one batch each: same result to fp32 round-off of
-    the merge order (far inside the bar), for bf16 and float16, head_dim 128 and 64, a
-    group of 16, and a batch with empty sequences in it."""
+    the merge order (far inside the bar), for bf16 and float16, head_dim 128 and 64,
+    groups of 16 and of 32 query heads (a cache head walked as two), and a batch with empty
+    sequences in it."""
     import torch
     from nanovllm_jax_amd import _lib, paged_attention
     from oracle.paged_attention_oracle import bf16_bits_to_f32
@@ -395,7 +396,8 @@ def test_balanced_split_whole_rows_equal_the_shared_rows_split():
     for seed, B, Hq, Hkv, D, lo, hi, dt in [(1, 64, 32, 8, 128, 1000, 1024, torch.bfloat16),
                                             (2, 128, 16, 8, 64, 400, 420, torch.float16),
                                             (3, 256, 32, 2, 128, 200, 224, torch.bfloat16),
-                                            (4, 128, 16, 16, 64, 0, 1200, torch.bfloat16)]:
+                                            (4, 128, 16, 16, 64, 0, 1200, torch.bfloat16),
+                                            (5, 128, 128, 4, 128, 300, 320, torch.float16)]:
         print(f"case both layouts seed={seed} B={B} Hq={Hq} Hkv={Hkv} D={D} {dt}", flush=True)
         rng = np.random.Generator(np.random.PCG64(seed))
         bs = 32
