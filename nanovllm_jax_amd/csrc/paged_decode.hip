@@ -1283,8 +1283,9 @@ __device__ __forceinline__ void merge_row(const DecodeArgs& a, uint4* lds, int b
 template <int D, bool F16, int VG = 0>
 __global__ __launch_bounds__(512) void paged_decode_balanced_kernel(DecodeArgs a, int batch,
                                                                     int num_wgs, int min_steps,
-                                                                    int hpw, int wr_hpw, int wr_tol,
-                                                                    int shift, int32_t* counters) {
+                                                                    int hpw, int wr_hpw, int wr_hpw_alt,
+                                                                    int wr_tol, int shift,
+                                                                    int32_t* counters) {
   using H = HeadDim<D>;
   constexpr int NW = 8;
   __shared__ uint4 k_tile[NW][kStep * H::kLdsRowPieces];
@@ -1367,11 +1368,6 @@ __global__ __launch_bounds__(512) void paged_decode_balanced_kernel(DecodeArgs a
   // wave of the launch reads the same lengths and takes the same decision.
   // -------------------------------------------------------------------------
   if (wr_hpw > 0 && total > 0) {
-    const int w_hpw = wr_hpw;
-    const int w_rps = a.num_kv_heads / w_hpw;       // a power of two (the host sees to it)
-    const int rps_shift = __builtin_ctz(w_rps);
-    const int rows = batch * w_rps;
-    const int rounds = (rows + num_wgs - 1) / num_wgs;
     // every wave writes all the lengths and step counts itself (the same values
     // from each), so no wave has to wait for another before it reads them back
     int key[kKeep];
@@ -1393,37 +1389,57 @@ __global__ __launch_bounds__(512) void paged_decode_balanced_kernel(DecodeArgs a
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
     __builtin_amdgcn_wave_barrier();
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-    // the largest number of steps any workgroup is dealt; steps_of_rank: the
-    // steps of the sequence of a given rank (wr_steps in the order of the batch,
-    // wr_sorted in the order by length)
-    auto largest_deal = [&](const int* steps_of_rank) {
-      int worst = 0;
-#pragma unroll
-      for (int w0 = 0; w0 < kMaxWholeRowWorkgroups; w0 += 64) {
-        const int w = w0 + lane;
-        int load = 0;
-        for (int t = 0; t < rounds; ++t) {
-          const int p = t * num_wgs + ((t & 1) ? num_wgs - 1 - w : w);
-          if (w < num_wgs && p < rows) load += steps_of_rank[p >> rps_shift];
+
+    // Two candidates: wr_hpw KV heads per workgroup and, when whole rows of
+    // that many heads cannot be dealt evenly enough, half as many (twice the
+    // rows, another round or more to pair long with short; fewer heads side by
+    // side stream a few percent slower, which is why it is second).
+    int w_hpw = 0, w_rps = 1, rps_shift = 0, rows = 0, rounds = 0;
+    bool whole_rows = false, sorted = false, ranked = false;
+    for (int candidate = 0; candidate < 2 && !whole_rows; ++candidate) {
+      w_hpw = candidate == 0 ? wr_hpw : wr_hpw_alt;
+      if (w_hpw <= 0) break;
+      w_rps = a.num_kv_heads / w_hpw;       // a power of two (the host sees to it)
+      rps_shift = __builtin_ctz(w_rps);
+      rows = batch * w_rps;
+      rounds = (rows + num_wgs - 1) / num_wgs;
+      // the largest number of steps any workgroup is dealt; steps_of_rank: the
+      // steps of the sequence of a given rank (wr_steps in the order of the
+      // batch, wr_sorted in the order by length)
+      auto largest_deal = [&](const int* steps_of_rank) {
+        int worst = 0;
+        for (int w0 = 0; w0 < num_wgs; w0 += 64) {
+          const int w = w0 + lane;
+          int load = 0;
+          for (int t = 0; t < rounds; ++t) {
+            const int p = t * num_wgs + ((t & 1) ? num_wgs - 1 - w : w);
+            if (w < num_wgs && p < rows) load += steps_of_rank[p >> rps_shift];
+          }
+          worst = max(worst, load);
         }
-        worst = max(worst, load);
+        return wave_max(worst);
+      };
+      const int64_t share = (int64_t)w_rps * total;   // num_wgs * a workgroup's share of the steps
+      const auto fits = [&](int load, int tol) {
+        return (int64_t)load * num_wgs * 256 <= share * (256 + tol);
+      };
+      // A row longer than the limit rules both orders out.  With one round
+      // every workgroup gets one row and the longest row decides.  With more
+      // rounds the order of the batch is only taken when it is as good as
+      // balanced (and only looked at when the lengths are within an eighth of
+      // each other); otherwise the order by length gets its chance.
+      if (!fits(longest, wr_tol)) continue;
+      sorted = false;
+      if (rounds == 1) {
+        whole_rows = true;
+        break;
       }
-      return wave_max(worst);
-    };
-    const int64_t budget = (int64_t)w_rps * total * (256 + wr_tol);   // 256 * num_wgs * the limit
-    const auto fits = [&](int load) { return (int64_t)load * num_wgs * 256 <= budget; };
-    // A row longer than the limit rules both orders out.  With one round every
-    // workgroup gets one row and the longest row decides.  With more rounds the
-    // order of the batch is only taken when it is as good as balanced (and only
-    // looked at when the lengths are within an eighth of each other); otherwise
-    // the order by length gets its chance.
-    bool whole_rows = fits(longest);
-    bool sorted = false;
-    if (whole_rows && rounds > 1) {
-      whole_rows = (longest - shortest) * 8 <= longest &&
-                   (int64_t)largest_deal(wr_steps) * num_wgs * 256 <=
-                       (int64_t)w_rps * total * (256 + min(wr_tol, kWholeRowTightTolerance));
-      if (!whole_rows) {
+      if ((longest - shortest) * 8 <= longest &&
+          fits(largest_deal(wr_steps), min(wr_tol, kWholeRowTightTolerance))) {
+        whole_rows = true;
+        break;
+      }
+      if (!ranked) {
         // Rank of every sequence by decreasing key: two threads per sequence
         // count, over half of the batch each, the keys above its own.  The keys
         // go through LDS (every wave writes all of them, the same values from
@@ -1456,9 +1472,10 @@ __global__ __launch_bounds__(512) void paged_decode_balanced_kernel(DecodeArgs a
           wr_sorted[above] = mine >> 8;
         }
         __syncthreads();
-        sorted = true;
-        whole_rows = fits(largest_deal(wr_sorted));
+        ranked = true;
       }
+      sorted = true;
+      whole_rows = fits(largest_deal(wr_sorted), wr_tol);
     }
     if (whole_rows) {
       const int w_parts = NW / w_hpw;
@@ -1883,7 +1900,7 @@ size_t counter_region_bytes(int64_t batch, int64_t kv_heads) {
 struct WorkspacePlan {
   int64_t records;  // partial records (one query head each)
   int max_chunks;   // fixed-chunk mode only
-  int num_wgs, hpw, wr_hpw, shift;  // balanced mode only
+  int num_wgs, hpw, wr_hpw, wr_hpw_alt, shift;  // balanced mode only
   size_t counter_bytes;
   size_t bytes;
 };
@@ -1907,15 +1924,27 @@ bool plan_workspace(int64_t batch, int64_t num_heads, int64_t head_dim, int64_t 
     while ((((axis >> plan->shift) + 2) * wgs * parts) >> 31) ++plan->shift;
     // The whole-row layout of the kernel (no partials at all) is offered when the
     // kernel keeps every length in registers and there is a row for every
-    // workgroup, with as many heads per workgroup as still give that (2 at
-    // least: with 1 the K/V stream of a large launch is a tenth slower).  It
-    // needs no workspace of its own.
-    plan->wr_hpw = 0;
+    // workgroup: with as many heads per workgroup as still give that, 2 at least
+    // (rows of 1 head are only worth it as the second choice: 32 equal sequences
+    // of 8192 positions take 167 us that way against 164 with the equal cut), and
+    // as a second choice with half as many heads, which gives the kernel another
+    // round or more of rows to pair long ones with short ones (64 sequences of
+    // 2048..6144 positions: 175 us with 1 head per workgroup, by length, against
+    // 180 with the equal cut; 128 of 2000..6000: 321 with 2 heads against 329).
+    // The layout needs no workspace of its own.
+    plan->wr_hpw = plan->wr_hpw_alt = 0;
+    const auto whole_rows_can_use = [&](int h) {
+      const int rps = h > 0 && num_kv_heads % h == 0 ? num_kv_heads / h : 0;
+      return rps > 0 && (rps & (rps - 1)) == 0 &&   // the kernel divides by shifting
+             batch * rps >= wgs;
+    };
     if (batch <= kKeptSequences && wgs <= kMaxWholeRowWorkgroups)
       for (int h = hpw; h >= 2; h /= 2)
         if (num_kv_heads % h == 0 && batch * (num_kv_heads / h) >= wgs) {
-          const int rps = num_kv_heads / h;
-          if ((rps & (rps - 1)) == 0) plan->wr_hpw = h;   // the kernel divides by shifting
+          if (whole_rows_can_use(h)) {
+            plan->wr_hpw = h;
+            if (whole_rows_can_use(h / 2)) plan->wr_hpw_alt = h / 2;
+          }
           break;
         }
     plan->max_chunks = 0;
@@ -1927,7 +1956,7 @@ bool plan_workspace(int64_t batch, int64_t num_heads, int64_t head_dim, int64_t 
   }
   const int64_t mc = (max_blocks * block_size + chunk - 1) / chunk;
   if (batch * mc > INT32_MAX) return false;
-  plan->num_wgs = plan->hpw = plan->wr_hpw = plan->shift = 0;
+  plan->num_wgs = plan->hpw = plan->wr_hpw = plan->wr_hpw_alt = plan->shift = 0;
   plan->max_chunks = (int)mc;
   plan->records = batch * mc * num_heads;
   plan->counter_bytes = 0;
@@ -2056,7 +2085,7 @@ int launch_decode(void* stream, const void* q, const void* k_cache, const void* 
     return rc == hipSuccess ? NVJ_OK : NVJ_ERR_LAUNCH;
   }
 
-  WorkspacePlan plan = {0, 1, 0, 0, 0, 0, 0, 0};
+  WorkspacePlan plan = {0, 1, 0, 0, 0, 0, 0, 0, 0};
   if (max_blocks > 0) {
     if (!plan_workspace(batch, num_heads, head_dim, max_blocks, block_size, num_kv_heads, chunk,
                         &plan))
@@ -2082,8 +2111,8 @@ int launch_decode(void* stream, const void* q, const void* k_cache, const void* 
 #define NVJ_LAUNCH_BALANCED(DV, F16V, VGV)                                                     \
   rc = nvj::launch(paged_decode_balanced_kernel<DV, F16V, VGV>, grid, dim3(512), s, a, batch, \
                    plan.num_wgs, kMinBalancedSteps, plan.hpw,                      \
-                   (phases & NVJ_PHASE_SHARED_ROWS) ? 0 : plan.wr_hpw, kWholeRowTolerance,    \
-                   plan.shift, counters)
+                   (phases & NVJ_PHASE_SHARED_ROWS) ? 0 : plan.wr_hpw, plan.wr_hpw_alt,       \
+                   kWholeRowTolerance, plan.shift, counters)
       if (loads_only) NVJ_LAUNCH_BALANCED(128, false, -1);
       else if (valu && group == 4) NVJ_LAUNCH_BALANCED(128, false, 4);
       else if (valu) NVJ_LAUNCH_BALANCED(128, false, 8);

@@ -274,37 +274,46 @@ def deals_whole_rows(ctx, num_kv_heads, table_positions, cus=256, tolerance=64, 
         hpw //= 2
     axis = (num_kv_heads // hpw) * B * max_steps
     wgs = min(cus, max(1, -(-axis // (8 // hpw))))
-    wr = 0
+
+    def usable(h):      # rows per sequence a power of two, a row for every workgroup
+        rps = num_kv_heads // h if h > 0 and num_kv_heads % h == 0 else 0
+        return rps > 0 and rps & (rps - 1) == 0 and B * rps >= wgs
+
+    candidates = []
     h = hpw
-    while B <= 256 and h >= 2:
+    while B <= 256 and wgs <= 256 and h >= 2:
         if num_kv_heads % h == 0 and B * (num_kv_heads // h) >= wgs:
-            rps = num_kv_heads // h
-            wr = h if rps & (rps - 1) == 0 else 0      # rows per sequence: a power of two
+            if usable(h):
+                candidates = [h] + ([h // 2] if usable(h // 2) else [])
             break
         h //= 2
     steps = _steps(ctx, table_positions)
-    if wr == 0 or steps.sum() == 0:
+    if steps.sum() == 0:
         return False, False
-    rps = num_kv_heads // wr
-    rows = B * rps
-    rounds = -(-rows // wgs)
+    by_length = np.argsort(-steps, kind="stable")
+    for h in candidates:
+        rps = num_kv_heads // h
+        rows = B * rps
+        rounds = -(-rows // wgs)
+        share = rps * int(steps.sum())
 
-    def largest(order):
-        load = np.zeros(wgs, np.int64)
-        for p in range(rows):
-            t, w = divmod(p, wgs)
-            load[wgs - 1 - w if t % 2 else w] += steps[order[p // rps]]
-        return int(load.max())
+        def largest(order):
+            load = np.zeros(wgs, np.int64)
+            for p in range(rows):
+                t, w = divmod(p, wgs)
+                load[wgs - 1 - w if t % 2 else w] += steps[order[p // rps]]
+            return int(load.max())
 
-    budget = rps * int(steps.sum()) * (256 + tolerance)
-    if int(steps.max()) * wgs * 256 > budget:          # one row alone is too much
-        return False, False
-    # the order of the batch: with several rows per workgroup only when all but even
-    first = budget if rounds == 1 else rps * int(steps.sum()) * (256 + min(tolerance, tight))
-    if largest(np.arange(B)) * wgs * 256 <= first:
-        return True, False
-    if rounds > 1 and largest(np.argsort(-steps, kind="stable")) * wgs * 256 <= budget:
-        return True, True
+        if int(steps.max()) * wgs * 256 > share * (256 + tolerance):   # one row alone is too much
+            continue
+        if rounds == 1:
+            return True, False
+        # the order of the batch: only when the lengths are close and the deal all but even
+        if (steps.max() - steps.min()) * 8 <= steps.max() and \
+                largest(np.arange(B)) * wgs * 256 <= share * (256 + min(tolerance, tight)):
+            return True, False
+        if largest(by_length) * wgs * 256 <= share * (256 + tolerance):
+            return True, True
     return False, False
 
 
@@ -338,8 +347,9 @@ def test_balanced_split_deals_whole_rows_when_that_is_balanced(name):
     workgroups within a quarter of an equal share, shares no row (the workspace stays
     untouched): equal lengths; lengths a few percent or a sixth apart; one short
     sequence among equal ones; lengths that only balance when long rows are paired with short ones
-    (the order by decreasing length, two and four rounds of rows).  It must not do so
-    when one long sequence, lengths a half apart or a log-uniform spread would leave
+    (the order by decreasing length, two and four rounds of rows).  Lengths a half apart only balance with half as many KV heads per
+    workgroup (twice the rows, paired by length): the kernel's second choice.  It must
+    not deal whole rows when one long sequence or a log-uniform spread would leave
     workgroups idle for long, and
     not when the caller forbids it.  Every case against the oracle, and the layout
     against the rule restated in deals_whole_rows."""
@@ -376,7 +386,7 @@ def test_balanced_split_deals_whole_rows_when_that_is_balanced(name):
     whole, by_length = deals_whole_rows(ctx, Hkv, bt.shape[1] * bs)
     expect = {"equal": (True, False), "within_tolerance": (True, False),
               "one_short": (True, False), "one_long": (False, False),
-              "a_sixth_apart": (True, False), "a_half_apart": (False, False),
+              "a_sixth_apart": (True, False), "a_half_apart": (True, True),
               "pairs_by_length": (True, True), "pairs_four_rounds": (True, True),
               "log_uniform": (False, False), "equal_forced_shared": (True, False)}[name]
     assert (whole, by_length) == expect, "the case does not exercise what its name says"
