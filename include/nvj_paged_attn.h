@@ -96,9 +96,9 @@ NVJ_API int nvj_store_kvcache_launch(void* stream,
  *               lengths.  Where whole (sequence, head group) rows can be dealt
  *               to the workgroups within a quarter of an equal share of the
  *               32-position steps (lengths equal or nearly so; or, taken by
- *               decreasing length, long rows that pair up with short ones), no
- *               row is shared between workgroups and the workspace is not
- *               touched (the launch is bound by the memory system as a whole,
+ *               decreasing length, long rows that pair up with short ones,
+ *               if need be with rows of half as many KV heads), no row is
+ *               shared between workgroups and the workspace is not touched (the launch is bound by the memory system as a whole,
  *               so an uneven deal costs far less than its unevenness, and
  *               less than sharing rows does).  Otherwise the steps of all rows, end to end, are cut
  *               into equal runs, one per wave; a row that fits one workgroup is
