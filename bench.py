@@ -240,11 +240,14 @@ def decode_step_record(steps, warmup, torch):
 MFMA_BF16_PEAK_TFLOPS = 2500.0
 
 
-def prefill_record(lens, prefix, steps, warmup, torch):
+def prefill_record(lens, prefix, steps, warmup, torch, zero_inputs=False):
     """Variable-length causal prefill attention at the Qwen3-8B head shape
     (Hq=32, Hkv=8, D=128): 8 prompts of 4096 tokens, packed.  Reports TFLOP/s
     (4 * Hq * D flop per visible (query, key) pair) against the dense bf16 MFMA
-    peak."""
+    peak.  `zero_inputs`: q, k and v all zero, a measuring aid: the kernel issues
+    the same instructions in the same number of cycles, but operands that never
+    toggle draw little power, so the chip holds its full clock and the figure shows
+    what the kernel's cycle count alone would give."""
     from nanovllm_jax_amd import paged_prefill_attention, variable_length_attention_prefill
     dev = torch.device("cuda:0")
     hq, hkv, d = 32, 8, 128
@@ -255,6 +258,8 @@ def prefill_record(lens, prefix, steps, warmup, torch):
     q = torch.randn((total, hq, d), generator=g, device=dev).to(torch.bfloat16)
     k = torch.randn((total, hkv, d), generator=g, device=dev).to(torch.bfloat16)
     v = torch.randn((total, hkv, d), generator=g, device=dev).to(torch.bfloat16)
+    if zero_inputs:
+        q.zero_(), k.zero_(), v.zero_()
     cu_t = torch.from_numpy(cu).to(dev)
     out = torch.empty_like(q)
     fn = lambda: variable_length_attention_prefill(q, k, v, cu_t, cu_t, scale=d ** -0.5, out=out)
@@ -273,6 +278,8 @@ def prefill_record(lens, prefix, steps, warmup, torch):
             used += n
         kc = torch.randn((sum(nblk), bs, hkv, d), generator=g, device=dev).to(torch.bfloat16)
         vc = torch.randn((sum(nblk), bs, hkv, d), generator=g, device=dev).to(torch.bfloat16)
+        if zero_inputs:
+            kc.zero_(), vc.zero_()
         cu_k = torch.from_numpy(np.concatenate([[0], np.cumsum(lens_k)]).astype(np.int32)).to(dev)
         bt_t = torch.from_numpy(bt).to(dev)
         fn = lambda: paged_prefill_attention(q, kc, vc, bt_t, cu_t, cu_k, d ** -0.5, out=out)
@@ -285,7 +292,8 @@ def prefill_record(lens, prefix, steps, warmup, torch):
     rec = {"metric": "prefill attention TFLOP/s (causal, varlen, Qwen3-8B head shape)",
            "value": round(tflops, 1), "unit": "TFLOP/s", "n_gpus": 1, "steps": steps,
            "warmup": warmup, "ms_per_step": round(wall, 4), "higher_is_better": True,
-           "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
+           "scaling": "weak", "vs_baseline": None, "dtype": "bf16",
+           "data": "all zeros (clock probe)" if zero_inputs else "synthetic",
            "config": {"workload": f"prefill: Hq={hq} Hkv={hkv} D={d}, prompt lengths {lens}" +
                                   (f" behind {prefix} cached positions each (paged cache)"
                                    if prefix > 0 else ""),
@@ -459,6 +467,9 @@ def main():
     ap.add_argument("--prefill-prefix", type=int, default=0,
                     help="with --prefill: cached positions in front of every prompt; keys and "
                          "values are then read from a paged cache")
+    ap.add_argument("--prefill-zero-inputs", action="store_true",
+                    help="with --prefill: q, k, v all zero (a clock probe: same instructions and "
+                         "cycles, little power, so the chip holds its full clock)")
     ap.add_argument("--decode-step", action="store_true",
                     help="time the whole-model decode step (config C5) instead of the "
                          "attention call; prints its own JSON line")
@@ -483,7 +494,7 @@ def main():
     if args.prefill:
         lens = [int(x) for x in args.prefill_lens.split(",")]
         print(json.dumps(prefill_record(lens, int(args.prefill_prefix), args.steps, args.warmup,
-                                        torch)), flush=True)
+                                        torch, zero_inputs=args.prefill_zero_inputs)), flush=True)
         return 0
 
     if args.copy_calibration:
