@@ -218,3 +218,40 @@ def test_reference_profile_shape_workload():
     assert (w.batch, w.num_heads, w.num_kv_heads, w.head_dim, w.block_size) == (64, 32, 32, 128, 256)
     assert np.array_equal(w.block_tables, np.arange(512, dtype=np.int32).reshape(64, 8))
     assert w.context_lens.min() >= 200 and w.context_lens.max() < 2048
+
+
+def test_bench_refuses_more_than_one_gpu():
+    """bench.py measures one GPU; asked for more it exits with a message that says so."""
+    import subprocess
+    import sys
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    r = subprocess.run([sys.executable, os.path.join(root, "bench.py"), "--gpus", "2"],
+                       capture_output=True, text=True, timeout=120)
+    assert r.returncode != 0
+    assert "ONE GPU" in (r.stdout + r.stderr)
+
+
+@pytest.mark.parametrize("name", ["C2_JITTER", "C2_SPREAD", "RAGGED_SHORT", "UNIFORM:12:100:900",
+                                  "LOGUNIFORM:7:16:5000:4:8"])
+def test_ragged_workload_metadata(name):
+    """The ragged bench workloads: lengths inside their stated range, every live page of
+    a block table distinct and inside the pool, slots pointing at the last position."""
+    from nanovllm_jax_amd.workloads import make_workload
+    w = make_workload(name)
+    again = make_workload(name)
+    assert np.array_equal(w.context_lens, again.context_lens)
+    assert np.array_equal(w.block_tables, again.block_tables)
+    lo, hi = {"C2_JITTER": (3840, 4096), "C2_SPREAD": (2048, 6144), "RAGGED_SHORT": (200, 2048),
+              "UNIFORM:12:100:900": (100, 900), "LOGUNIFORM:7:16:5000:4:8": (16, 5000)}[name]
+    assert w.context_lens.min() >= lo and w.context_lens.max() <= hi
+    nblk = -(-w.context_lens.astype(np.int64) // w.block_size)
+    live = np.concatenate([w.block_tables[b, :n] for b, n in enumerate(nblk)])
+    assert live.min() >= 0 and live.max() < w.num_blocks
+    assert len(np.unique(live)) == len(live)
+    for b, n in enumerate(nblk):
+        assert (w.block_tables[b, n:] == -1).all()
+        last = int(w.context_lens[b]) - 1
+        assert w.slot_mapping[b] == w.block_tables[b, last // w.block_size] * w.block_size + \
+            last % w.block_size
+    if name.startswith("LOGUNIFORM"):
+        assert (w.num_kv_heads, w.num_heads) == (4, 8)
