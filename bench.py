@@ -416,8 +416,12 @@ def others_block(args, torch, dev):
 
     def prefill():
         r = prefill_record([4096] * 8, 0, max(5, st // 5), 2, torch)
+        # the same launch on all-zero inputs: same cycles at the chip's full clock
+        z = prefill_record([4096] * 8, 0, max(5, st // 5), 2, torch, zero_inputs=True)
         return {"TFLOP/s": r["value"], "pct_of_mfma_bf16_peak": round(100 * r["roofline"]["frac"], 2),
-                "us_per_call": r["roofline"]["kernel_us"], "workload": r["config"]["workload"]}
+                "us_per_call": r["roofline"]["kernel_us"],
+                "TFLOP/s_on_zero_inputs_clock_probe": z["value"],
+                "workload": r["config"]["workload"]}
     run("prefill_8x4096", prefill)
 
     def step():
