@@ -408,7 +408,6 @@ __global__ __launch_bounds__(kWaves * 64, kGroups <= 2 ? 2 : 1) void prefill_att
   const int r = lane & 15;
   const int kg = lane >> 4;
   const const_i32_ptr cu_q = (const_i32_ptr)(uintptr_t)a.cu_q;
-  const const_i32_ptr cu_k = (const_i32_ptr)(uintptr_t)a.cu_k;
 
   // Work item -> workgroup, XCD-aware.  Consecutive workgroup ids land on
   // different XCDs (8 of them, each with its own L2), so the work list is cut
@@ -427,25 +426,60 @@ __global__ __launch_bounds__(kWaves * 64, kGroups <= 2 ? 2 : 1) void prefill_att
   const int in_kv = item - kvh * per_kv_head;
   const int tile_id = num_tiles_bound - 1 - in_kv / a.group;
   const int head = kvh * a.group + in_kv % a.group;
+  // The sequence that owns query tile tile_id: 64 sequences at a time, one per
+  // lane, the lengths of 256 sequences fetched together (one round trip per 256
+  // sequences whatever the batch; a loop over the sequences one by one cost a
+  // batch of 128 short prompts more than its tiles).
   int seq = -1, q0 = 0;
+  int q_base = 0, len_q = 0, k_first = 0, k_count = 0;   // of that sequence, from the same loads
   {
-    int before = 0;
-    for (int s = 0; s < a.batch; ++s) {
-      const int len = cu_q[s + 1] - cu_q[s];
-      const int nt = (max(len, 0) + kBM - 1) / kBM;
-      if (tile_id < before + nt) {
-        seq = s;
-        q0 = (tile_id - before) * kBM;
-        break;
+    int before = 0;   // tiles of the sequences in front of this group of 64
+    for (int base = 0; base < a.batch && seq < 0; base += 256) {
+      int nt4[4], qb4[4], ql4[4], kb4[4], kl4[4];
+#pragma unroll
+      for (int k = 0; k < 4; ++k) {
+        const int s = min(base + 64 * k + lane, a.batch - 1);
+        qb4[k] = a.cu_q[s];
+        ql4[k] = a.cu_q[s + 1] - qb4[k];
+        kb4[k] = a.cu_k[s];
+        kl4[k] = a.cu_k[s + 1] - kb4[k];
+        nt4[k] = base + 64 * k + lane < a.batch ? (max(ql4[k], 0) + kBM - 1) / kBM : 0;
       }
-      before += nt;
+#pragma unroll
+      for (int k = 0; k < 4; ++k) {
+        if (base + 64 * k < a.batch && seq < 0) {
+          const int nt = nt4[k];
+          int incl = nt;   // tiles up to and including this lane's sequence
+#pragma unroll
+          for (int d = 1; d < 64; d <<= 1) {
+            const int up = __shfl_up(incl, d, 64);
+            if (lane >= d) incl += up;
+          }
+          const unsigned long long hit =
+              __ballot(nt > 0 && tile_id >= before + incl - nt && tile_id < before + incl);
+          if (hit != 0ull) {
+            const int src = __builtin_ctzll(hit);
+            seq = base + 64 * k + src;
+            q0 = (tile_id - before - __shfl(incl - nt, src, 64)) * kBM;
+            q_base = __shfl(qb4[k], src, 64);
+            len_q = __shfl(ql4[k], src, 64);
+            k_first = __shfl(kb4[k], src, 64);
+            k_count = __shfl(kl4[k], src, 64);
+          }
+          before += __shfl(incl, 63, 64);
+        }
+      }
     }
+    seq = __builtin_amdgcn_readfirstlane(seq);
+    q0 = __builtin_amdgcn_readfirstlane(q0);
+    q_base = __builtin_amdgcn_readfirstlane(q_base);
+    len_q = __builtin_amdgcn_readfirstlane(len_q);
+    k_first = __builtin_amdgcn_readfirstlane(k_first);
+    k_count = __builtin_amdgcn_readfirstlane(k_count);
   }
   if (seq < 0) return;   // beyond the real number of tiles
-  const int q_base = cu_q[seq], len_q = cu_q[seq + 1] - q_base;
-  const int k_base = PAGED ? 0 : cu_k[seq];
-  const int len_k = PAGED ? min(max(cu_k[seq + 1] - cu_k[seq], 0), a.max_blocks * a.block_size)
-                          : max(cu_k[seq + 1] - k_base, 0);
+  const int k_base = PAGED ? 0 : k_first;
+  const int len_k = PAGED ? min(max(k_count, 0), a.max_blocks * a.block_size) : max(k_count, 0);
   // key position of query row 0: rows are the tail of the sequence when paged
   const int off = PAGED ? max(len_k - len_q, 0) : 0;
   const int q_end = min(q0 + kBM, len_q);           // rows [q0, q_end) are real

@@ -45,6 +45,28 @@ def test_prefill_ragged_batch(Hq, Hkv):
         assert np.array_equal(got[cu_q[i]], np.repeat(v[cu_k[i]], G, axis=0))
 
 
+@pytest.mark.parametrize("batch", [65, 130, 300, 600])
+def test_prefill_batches_of_many_short_prompts(batch):
+    """More sequences than the 64 a wave looks at together, and than the 256 whose
+    lengths it fetches in one go, when it finds the sequence of a query tile: short
+    prompts, empty ones and a few longer than a tile among them."""
+    print(f"case prefill many prompts batch={batch}", flush=True)
+    from oracle.paged_attention_oracle import variable_length_attention_prefill_ref
+    rng = np.random.Generator(np.random.PCG64(700 + batch))
+    lens = rng.integers(0, 41, size=batch)
+    lens[rng.integers(0, batch, size=5)] = [129, 257, 128, 1, 300]
+    lens[[0, 63, 64, batch - 1]] = [3, 130, 0, 131]
+    lens = [int(x) for x in lens]
+    q, k, v, cu_q, cu_k = _problem(710 + batch, lens, lens, 4, 2)
+    scale = 128 ** -0.5
+    want = variable_length_attention_prefill_ref(q, k, v, cu_q, cu_k, scale)
+    got = run_hip(q, k, v, cu_q, cu_k, scale)
+    assert_close_bf16(got, want, what=f"prefill {batch} prompts")
+    for i in range(batch):                        # first row of a sequence == its first V row
+        if lens[i] > 0:
+            assert np.array_equal(got[cu_q[i]], np.repeat(v[cu_k[i]], 2, axis=0)), i
+
+
 def test_prefill_reference_smoke_lengths():
     """Sequence lengths of the reference's prefill smoke test
     (test_mosaic_kernels.py:90-159): 512, 768, 1024, 1536; Hq=32, Hkv=8, D=128."""
