@@ -424,27 +424,43 @@ __global__ __launch_bounds__(kWaves * 64, kGroups <= 2 ? 2 : 1) void prefill_att
   const int per_kv_head = num_tiles_bound * a.group;
   const int kvh = item / per_kv_head;
   const int in_kv = item - kvh * per_kv_head;
-  const int tile_id = num_tiles_bound - 1 - in_kv / a.group;
   const int head = kvh * a.group + in_kv % a.group;
-  // The sequence that owns query tile tile_id: 64 sequences at a time, one per
-  // lane, the lengths of 256 sequences fetched together (one round trip per 256
-  // sequences whatever the batch; a loop over the sequences one by one cost a
-  // batch of 128 short prompts more than its tiles).
+  // Query tiles are numbered sequence by sequence.  A wave looks at 64 sequences
+  // at a time, one per lane, with the offsets of 256 sequences fetched together
+  // (one round trip per 256 sequences; a loop over the sequences one by one cost
+  // a batch of 128 short prompts more than its tiles).  First the real number of
+  // tiles: the work list was sized for a bound, and the items beyond the real
+  // tiles sit at its end, where they delay nothing.  The real tiles are walked
+  // from the last one down (the later tiles of a sequence have more keys).
+  int nt4[4], qb4[4], ql4[4], kb4[4], kl4[4];
+  auto load_offsets = [&](int base) {
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      const int s = min(base + 64 * k + lane, a.batch - 1);
+      qb4[k] = a.cu_q[s];
+      ql4[k] = a.cu_q[s + 1] - qb4[k];
+      kb4[k] = a.cu_k[s];
+      kl4[k] = a.cu_k[s + 1] - kb4[k];
+      nt4[k] = base + 64 * k + lane < a.batch ? (max(ql4[k], 0) + kBM - 1) / kBM : 0;
+    }
+  };
+  int real_tiles = 0;
+  for (int base = 0; base < a.batch; base += 256) {
+    load_offsets(base);
+    int sum = nt4[0] + nt4[1] + nt4[2] + nt4[3];
+#pragma unroll
+    for (int d = 1; d < 64; d <<= 1) sum += __shfl_xor(sum, d, 64);
+    real_tiles += sum;
+  }
+  real_tiles = __builtin_amdgcn_readfirstlane(real_tiles);
+  if (in_kv / a.group >= real_tiles) return;   // beyond the real number of tiles
+  const int tile_id = real_tiles - 1 - in_kv / a.group;
   int seq = -1, q0 = 0;
   int q_base = 0, len_q = 0, k_first = 0, k_count = 0;   // of that sequence, from the same loads
   {
     int before = 0;   // tiles of the sequences in front of this group of 64
     for (int base = 0; base < a.batch && seq < 0; base += 256) {
-      int nt4[4], qb4[4], ql4[4], kb4[4], kl4[4];
-#pragma unroll
-      for (int k = 0; k < 4; ++k) {
-        const int s = min(base + 64 * k + lane, a.batch - 1);
-        qb4[k] = a.cu_q[s];
-        ql4[k] = a.cu_q[s + 1] - qb4[k];
-        kb4[k] = a.cu_k[s];
-        kl4[k] = a.cu_k[s + 1] - kb4[k];
-        nt4[k] = base + 64 * k + lane < a.batch ? (max(ql4[k], 0) + kBM - 1) / kBM : 0;
-      }
+      if (a.batch > 256) load_offsets(base);   // (a smaller batch is still in registers)
 #pragma unroll
       for (int k = 0; k < 4; ++k) {
         if (base + 64 * k < a.batch && seq < 0) {
@@ -477,7 +493,7 @@ __global__ __launch_bounds__(kWaves * 64, kGroups <= 2 ? 2 : 1) void prefill_att
     k_first = __builtin_amdgcn_readfirstlane(k_first);
     k_count = __builtin_amdgcn_readfirstlane(k_count);
   }
-  if (seq < 0) return;   // beyond the real number of tiles
+  if (seq < 0) return;   // (cannot happen: tile_id is a real tile)
   const int k_base = PAGED ? 0 : k_first;
   const int len_k = PAGED ? min(max(k_count, 0), a.max_blocks * a.block_size) : max(k_count, 0);
   // key position of query row 0: rows are the tail of the sequence when paged
